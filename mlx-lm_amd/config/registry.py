@@ -7,7 +7,7 @@ MODEL_REMAPPING = {}
 
 _REGISTRY = {}
 _BUILTIN = {"gpt2": "mlx_lm_amd.models.gpt2", "pafutar": "mlx_lm_amd.models.pafutar",
-            "ruzolorn": "mlx_lm_amd.models.ruzolorn"}
+            "ruzolorn": "mlx_lm_amd.models.ruzolorn", "zatinex": "mlx_lm_amd.models.zatinex"}
 
 
 def register_model(model_type, model_cls, args_cls):

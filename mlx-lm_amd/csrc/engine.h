@@ -147,6 +147,7 @@ int eng_rows_split_from(void);
 #define ENG_SETTLES_PENDING 2
 #define ENG_HANDLES_PENDING 4
 #define ENG_READS_AHEAD 8
+#define ENG_WANTS_STATE 16  // a mixer: it is handed the run's state slot beside its cache slot
 
 typedef struct EngPart EngPart;
 
@@ -180,6 +181,9 @@ int eng_norm_forward(EngPart* norm, EngCtx* ctx, const EngMat* x, const int* row
 int eng_mixer_forward(EngPart* mixer, EngCtx* ctx, const EngValue* x, const EngMat* residual, int cache_slot,
                       int writes_cache);
 int eng_ffn_forward(EngPart* ffn, EngCtx* ctx, const EngValue* x, const EngMat* residual);
+// attention of the step's queries over a slot's pages, the kernels chosen as the attention part does
+int eng_attend(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads, int head_dim,
+               int window, float scale, int array_base);
 int eng_embedding_forward(EngPart* embedding, EngCtx* ctx, const EngMat* out, EngPart* positions);
 int eng_head_forward(EngPart* head, EngCtx* ctx, const EngValue* x, const EngMat* out);
 int eng_settle(EngCtx* ctx);

@@ -577,11 +577,15 @@ struct PyPosition : Position {
 
 struct PyMixer : Mixer {
   int id;
-  PyMixer(int i, int flags) : id(i) { accepts_lazy = false, (void)flags; }
+  PyMixer(int i, int flags) : id(i) { accepts_lazy = false, wants_state = (flags & ENG_WANTS_STATE) != 0; }
   int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes) override {
+    return forward_with_state(ctx, x, residual, slot, writes, -1);
+  }
+  int forward_with_state(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes,
+                         int state_slot) override {
     EngCall c = {};
     TRY(materialize(ctx, x, &c.x));
-    c.residual = residual, c.cache_slot = slot, c.writes_cache = writes;
+    c.residual = residual, c.cache_slot = slot, c.writes_cache = writes, c.state_slot = state_slot;
     return call_python(id, ENG_CB_MIXER, ctx, &c);
   }
 };
@@ -893,17 +897,22 @@ struct PreNormBlock : Block {
     return norm->forward(ctx, h, nullptr, 0, lazy, norm->reads_ahead ? first : nullptr, may_pack, x);
   }
 
-  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int) override {
+  // (a layer may have no feed-forward: ffn and ffn_norm are then null; a mixer that keeps state
+  // beside its pages gets the run's state slot)
+  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int state_slot) override {
     const size_t mark = ctx->scratch->offset;
     EngValue x;
     TRY(normed(ctx, mixer_norm, h, mixer->accepts_lazy, mixer->accepts_packed, mixer->first_weight, &x));
     // (a mixer whose kernels leave CUs idle may have them read the weights that come after its own)
-    ctx->read_ahead = ffn->first_weight;
-    int rc = mixer->forward(ctx, x, h, slot, writes);
+    ctx->read_ahead = ffn ? ffn->first_weight : nullptr;
+    int rc = mixer->wants_state ? mixer->forward_with_state(ctx, x, h, slot, writes, state_slot)
+                                : mixer->forward(ctx, x, h, slot, writes);
     ctx->read_ahead = nullptr;
     if (rc) return rc;
-    TRY(normed(ctx, ffn_norm, h, ffn->accepts_lazy, ffn->accepts_packed, ffn->first_weight, &x));
-    TRY(ffn->forward(ctx, x, h));
+    if (ffn) {
+      TRY(normed(ctx, ffn_norm, h, ffn->accepts_lazy, ffn->accepts_packed, ffn->first_weight, &x));
+      TRY(ffn->forward(ctx, x, h));
+    }
     ctx->scratch->offset = mark;
     return 0;
   }
@@ -1099,9 +1108,11 @@ extern "C" EngPart* eng_make_pre_norm_block(EngPart* mixer_norm, EngPart* mixer,
   PreNormBlock* b = new PreNormBlock();
   b->mixer_norm = as<Norm>(mixer_norm, KIND_NORM, "eng_make_pre_norm_block");
   b->mixer = as<Mixer>(mixer, KIND_MIXER, "eng_make_pre_norm_block");
-  b->ffn_norm = as<Norm>(ffn_norm, KIND_NORM, "eng_make_pre_norm_block");
-  b->ffn = as<FeedForward>(ffn, KIND_FFN, "eng_make_pre_norm_block");
-  if (!b->mixer_norm || !b->mixer || !b->ffn_norm || !b->ffn) {
+  b->ffn_norm = ffn_norm ? as<Norm>(ffn_norm, KIND_NORM, "eng_make_pre_norm_block") : nullptr;
+  b->ffn = ffn ? as<FeedForward>(ffn, KIND_FFN, "eng_make_pre_norm_block") : nullptr;
+  if (!b->mixer_norm || !b->mixer || (ffn_norm && !b->ffn_norm) || (ffn && !b->ffn) || !ffn != !ffn_norm) {
+    if (b->mixer_norm && b->mixer && !ffn != !ffn_norm)
+      snprintf(g_err, sizeof(g_err), "eng_make_pre_norm_block: a feed-forward and its norm, or neither");
     delete b;
     return nullptr;
   }
@@ -1175,6 +1186,27 @@ extern "C" int eng_mixer_forward(EngPart* mixer, EngCtx* ctx, const EngValue* x,
                                  int cache_slot, int writes_cache) {
   Mixer* m = as<Mixer>(mixer, KIND_MIXER, "eng_mixer_forward");
   return m ? m->forward(ctx, *x, *residual, cache_slot, writes_cache != 0) : 1;
+}
+
+// Causal attention of this step's queries over the pages of cache slot `slot`, with the choice
+// among the attention kernels that the built-in attention part makes (rows to the decode kernels,
+// portions to the tile kernels, by the step's work lists from `array_base` on): for a mixer that
+// prepares queries, keys and values in its own way and wants only this.
+extern "C" int eng_attend(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads,
+                          int head_dim, int window, float scale, int array_base) {
+  if (!out || !q || n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads)
+    FAIL("eng_attend: %d query heads over %d key heads", n_heads, n_kv_heads);
+  if (array_base < 0 || array_base + ARR_ROWS_ARE_REQUESTS >= ENG_MAX_ARRAYS)
+    FAIL("eng_attend: array ids from %d do not fit", array_base);
+  if (q->cols != n_heads * head_dim || out->cols != q->cols || out->rows != q->rows || out->dtype != q->dtype)
+    FAIL("eng_attend: queries and output are [tokens, %d] of one dtype", n_heads * head_dim);
+  Attention a;
+  a.width = 0, a.n_heads = n_heads, a.n_kv_heads = n_kv_heads, a.head_dim = head_dim, a.window = window;
+  a.scale = scale, a.q_width = n_heads * head_dim, a.kv_width = n_kv_heads * head_dim, a.array_base = array_base;
+  a.qkv_w = EngWeight{}, a.out_w = EngWeight{}, a.qkv_b = a.out_b = nullptr, a.position = nullptr;
+  EngScatter kv;
+  TRY(a.scatter_for(ctx, slot, &kv));
+  return a.attend(ctx, *out, *q, kv, false);
 }
 
 extern "C" int eng_ffn_forward(EngPart* ffn, EngCtx* ctx, const EngValue* x, const EngMat* residual) {

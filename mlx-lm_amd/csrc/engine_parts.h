@@ -57,12 +57,20 @@ struct Position : EngPart {
 // can_overwrite: the part is able to write its output into `residual` instead of adding to it;
 // an arrangement that wants the output by itself (a sum that is normed afterwards) then sets
 // `overwrite` on the parts it owns, and hands the others rows of zeros.
+// wants_state: the mixer keeps per-request state beside its pages (the inputs of a short
+// convolution ahead of its attention, say); the arrangement then calls forward_with_state with
+// the run's state slot.
 struct Mixer : EngPart {
   bool accepts_lazy = false, accepts_packed = false;
   bool can_overwrite = false, overwrite = false;
+  bool wants_state = false;
   const EngWeight* first_weight = nullptr;
   Mixer() : EngPart(KIND_MIXER) {}
   virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes) = 0;
+  virtual int forward_with_state(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes,
+                                 int /*state_slot*/) {
+    return forward(ctx, x, residual, slot, writes);
+  }
 };
 
 struct FeedForward : EngPart {

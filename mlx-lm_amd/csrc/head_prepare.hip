@@ -1,0 +1,219 @@
+// What lies between a projection and the attention (or recurrence) that reads its heads, and
+// between the attention and the output projection, for mixers that shape their heads in ways of
+// their own.  Everything is 32-bit inside; the sources are the projections' float rows.
+//
+//   causal_conv     y[t, c] = act(b[c] + sum_j w[c, j] u[t - taps + 1 + j, c]) over a request's own
+//                   tokens; inputs of earlier steps come from the request's state row ([taps - 1, C],
+//                   the latest last, zero at a request's start), which conv_state_update
+//                   (linear_state.hip) brings up to date afterwards.  With `single` (every request
+//                   brings one token) the kernel moves the state up itself.
+//   head_prepare    a wave a (row, head): the head's `dim` columns from a float row; RMS norm over
+//                   the first `norm_dim` of them (times a weight of norm_dim values shared by all
+//                   heads, or none); rotation of the `rot_dims` columns from `rot_off` on by
+//                   position * inv_freq[i], pairs (2i, 2i + 1) or (i, i + rot_dims / 2), cos and
+//                   sin times `rot_mult`; then the head goes to `copies` places: copy c of head h
+//                   to column dst_head[c * n_heads + h] * dst_stride of the output row (h itself
+//                   without a table), zeros from `dim` up to `dst_fill` columns.
+//   diff_combine    o = a1 - lambda a2 per head, where a1 and a2 are two heads of an attention's
+//                   output (tables say which), divided by its root mean square and multiplied by
+//                   `mult`.
+//   head_gate       x[t, h, :] *= sigmoid(g[t, h]), in place.
+#include "common.h"
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+
+// Thread (token row, channel).
+__global__ __launch_bounds__(256) void causal_conv_kernel(const float* __restrict__ u, int ldu, int col,
+                                                          const float* __restrict__ w, const float* __restrict__ b,
+                                                          int taps, int C, int act, float* __restrict__ state,
+                                                          size_t state_stride, size_t conv_offset,
+                                                          const int* __restrict__ token_req,
+                                                          const int* __restrict__ seq_start,
+                                                          const int* __restrict__ slot_ids, float* __restrict__ y,
+                                                          int ldy, int single) {
+  const int c = blockIdx.y * 256 + threadIdx.x, row = blockIdx.x;
+  if (c >= C) return;
+  const int req = token_req[row], local = row - seq_start[req];
+  float* old = state + (size_t)slot_ids[req] * state_stride + conv_offset;  // [taps - 1, C], the latest last
+  float acc = b ? b[c] : 0.f;
+  for (int j = taps - 1; j >= 0; --j) {  // the oldest input first
+    const int at = local - j;
+    const float in = at >= 0 ? u[(size_t)(row - j) * ldu + col + c] : old[(size_t)(taps - 1 + at) * C + c];
+    acc += w[(size_t)c * taps + (taps - 1 - j)] * in;
+    // every request brings one token: this thread alone reads and writes its request's inputs
+    // of channel c, so it moves them up by one as it goes (the oldest first)
+    if (single && j < taps - 1) old[(size_t)(taps - 2 - j) * C + c] = in;
+  }
+  y[(size_t)row * ldy + c] = act ? silu_f(acc) : acc;
+}
+
+struct PrepareArgs {
+  const float* src;
+  int lds, src_col, src_stride;  // head h at column src_col + h * src_stride
+  int n_rows, n_heads, dim;
+  int norm_dim;
+  const float* norm_w;  // [norm_dim] or null
+  float eps;
+  int rot_off, rot_dims, interleaved;
+  const float* inv_freq;  // [rot_dims / 2]
+  float rot_mult;
+  const int* positions;
+  void* dst;
+  int ldd, dst_stride, dst_fill, copies;
+  const int* dst_head;  // [copies, n_heads] or null
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void head_prepare_kernel(PrepareArgs a) {
+  const int lane = threadIdx.x & 63;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long)a.n_rows * a.n_heads) return;  // whole waves leave; no barrier follows
+  const int row = (int)(item / a.n_heads), h = (int)(item % a.n_heads);
+  const float* s = a.src + (size_t)row * a.lds + a.src_col + (size_t)h * a.src_stride;
+  float rstd = 1.f;
+  if (a.norm_dim > 0) {
+    float q = 0.f;
+    for (int k = lane; k < a.norm_dim; k += 64) q += s[k] * s[k];
+    rstd = 1.0f / sqrtf(wave_sum(q) / (float)a.norm_dim + a.eps);
+  }
+  const float pos = a.rot_dims ? (float)a.positions[row] : 0.f;
+  const int half = a.rot_dims / 2;
+  for (int k = lane; k < a.dst_fill; k += 64) {
+    float v = 0.f;
+    if (k < a.dim) {
+      const int rel = k - a.rot_off;
+      auto at = [&](int c) { return c < a.norm_dim ? s[c] * rstd * (a.norm_w ? a.norm_w[c] : 1.f) : s[c]; };
+      v = at(k);
+      if (rel >= 0 && rel < a.rot_dims) {
+        int i, partner;
+        bool first;  // this column is the pair's first member
+        if (a.interleaved)
+          i = rel >> 1, first = !(rel & 1), partner = first ? k + 1 : k - 1;
+        else
+          first = rel < half, i = first ? rel : rel - half, partner = first ? k + half : k - half;
+        float sn, cs;
+        sincosf(pos * a.inv_freq[i], &sn, &cs);
+        sn *= a.rot_mult, cs *= a.rot_mult;
+        const float other = at(partner);
+        v = first ? v * cs - other * sn : v * cs + other * sn;
+      }
+    }
+    for (int c = 0; c < a.copies; ++c) {
+      const int dh = a.dst_head ? a.dst_head[c * a.n_heads + h] : h;
+      ((T*)a.dst)[(size_t)row * a.ldd + (size_t)dh * a.dst_stride + k] = from_f32<T>(v);
+    }
+  }
+}
+
+// A wave a (row, head).
+template <typename T>
+__global__ __launch_bounds__(256) void diff_combine_kernel(const T* __restrict__ att, int lda, int head_stride,
+                                                           const int* __restrict__ first, const int* __restrict__ second,
+                                                           float lambda, float mult, float eps, int n_rows, int n_heads,
+                                                           int vdim, T* __restrict__ out, int ldo) {
+  const int lane = threadIdx.x & 63;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long)n_rows * n_heads) return;
+  const int row = (int)(item / n_heads), h = (int)(item % n_heads);
+  const T* a1 = att + (size_t)row * lda + (size_t)first[h] * head_stride;
+  const T* a2 = att + (size_t)row * lda + (size_t)second[h] * head_stride;
+  float q = 0.f;
+  for (int k = lane; k < vdim; k += 64) {
+    const float o = to_f32(a1[k]) - lambda * to_f32(a2[k]);
+    q += o * o;
+  }
+  const float f = mult / sqrtf(wave_sum(q) / (float)vdim + eps);
+  for (int k = lane; k < vdim; k += 64)
+    out[(size_t)row * ldo + (size_t)h * vdim + k] = from_f32<T>((to_f32(a1[k]) - lambda * to_f32(a2[k])) * f);
+}
+
+// Thread (row, column).
+template <typename T>
+__global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ x, int ldx, int head_stride, int n_heads,
+                                                        const float* __restrict__ g, int ldg, int n_rows) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  const int width = n_heads * head_stride;
+  if (e >= (long)n_rows * width) return;
+  const int row = (int)(e / width), c = (int)(e % width);
+  const float z = g[(size_t)row * ldg + c / head_stride];
+  T* p = x + (size_t)row * ldx + c;
+  *p = from_f32<T>(to_f32(*p) / (1.0f + expf(-z)));
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+extern "C" int causal_conv(const float* u, int ldu, int col, const float* w, const float* b, int taps, int C, int act,
+                           float* state, size_t state_stride, size_t conv_offset, const int* token_req,
+                           const int* seq_start, const int* slot_ids, float* y, int ldy, int n_tokens, int single,
+                           hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (!u || !w || !state || !token_req || !seq_start || !slot_ids || !y) FAIL("causal_conv: null pointer");
+  if (taps < 1 || C <= 0 || col < 0 || col + C > ldu || ldy < C)
+    FAIL("causal_conv: %d taps, %d channels from column %d, rows of %d and %d", taps, C, col, ldu, ldy);
+  dim3 grid(n_tokens, (C + 255) / 256), block(256);
+  hipLaunchKernelGGL(causal_conv_kernel, grid, block, 0, stream, u, ldu, col, w, b, taps, C, act, state, state_stride,
+                     conv_offset, token_req, seq_start, slot_ids, y, ldy, single);
+  CHECK_LAUNCH("causal_conv");
+  return 0;
+}
+
+extern "C" int head_prepare(const PrepareArgs* args, int dst_dtype, hipStream_t stream) {
+  const PrepareArgs& a = *args;
+  if (a.n_rows <= 0 || a.n_heads <= 0) return 0;
+  if (!a.src || !a.dst) FAIL("head_prepare: null pointer");
+  if (a.dim <= 0 || a.src_col < 0 || a.src_col + (long)(a.n_heads - 1) * a.src_stride + a.dim > a.lds)
+    FAIL("head_prepare: %d heads of %d columns, %d apart from column %d, in rows of %d", a.n_heads, a.dim, a.src_stride,
+         a.src_col, a.lds);
+  if (a.norm_dim < 0 || a.norm_dim > a.dim) FAIL("head_prepare: a norm over %d of %d columns", a.norm_dim, a.dim);
+  if (a.rot_dims && (a.rot_dims % 2 || a.rot_off < 0 || a.rot_off + a.rot_dims > a.dim || !a.inv_freq || !a.positions))
+    FAIL("head_prepare: %d turning columns from %d in a head of %d", a.rot_dims, a.rot_off, a.dim);
+  if (a.copies < 1 || a.dst_fill < a.dim || a.dst_fill > a.dst_stride)
+    FAIL("head_prepare: %d copies, %d columns filled of %d, a head of %d", a.copies, a.dst_fill, a.dst_stride, a.dim);
+  if (!a.dst_head && (a.copies != 1 || (long)(a.n_heads - 1) * a.dst_stride + a.dst_fill > a.ldd))
+    FAIL("head_prepare: the heads do not fit rows of %d", a.ldd);
+  if (dst_dtype != DT_F32 && dst_dtype != DT_BF16) FAIL("head_prepare: unknown dtype code %d", dst_dtype);
+  const long items = (long)a.n_rows * a.n_heads;
+  dim3 grid((unsigned)((items + 3) / 4)), block(256);
+  if (dst_dtype == DT_F32)
+    hipLaunchKernelGGL(head_prepare_kernel<float>, grid, block, 0, stream, a);
+  else
+    hipLaunchKernelGGL(head_prepare_kernel<bf16>, grid, block, 0, stream, a);
+  CHECK_LAUNCH("head_prepare");
+  return 0;
+}
+
+extern "C" int diff_combine(const void* att, int lda, int head_stride, const int* first, const int* second, float lambda,
+                            float mult, float eps, int n_rows, int n_heads, int vdim, void* out, int ldo, int dtype,
+                            hipStream_t stream) {
+  if (n_rows <= 0 || n_heads <= 0) return 0;
+  if (!att || !first || !second || !out) FAIL("diff_combine: null pointer");
+  if (vdim <= 0 || vdim > head_stride || ldo < n_heads * vdim) FAIL("diff_combine: values of %d in heads of %d, rows of %d", vdim, head_stride, ldo);
+  if (dtype != DT_F32 && dtype != DT_BF16) FAIL("diff_combine: unknown dtype code %d", dtype);
+  const long items = (long)n_rows * n_heads;
+  dim3 grid((unsigned)((items + 3) / 4)), block(256);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(diff_combine_kernel<float>, grid, block, 0, stream, (const float*)att, lda, head_stride, first, second,
+                       lambda, mult, eps, n_rows, n_heads, vdim, (float*)out, ldo);
+  else
+    hipLaunchKernelGGL(diff_combine_kernel<bf16>, grid, block, 0, stream, (const bf16*)att, lda, head_stride, first, second,
+                       lambda, mult, eps, n_rows, n_heads, vdim, (bf16*)out, ldo);
+  CHECK_LAUNCH("diff_combine");
+  return 0;
+}
+
+extern "C" int head_gate(void* x, int ldx, int head_stride, int n_heads, const float* g, int ldg, int n_rows, int dtype,
+                         hipStream_t stream) {
+  if (n_rows <= 0 || n_heads <= 0) return 0;
+  if (!x || !g) FAIL("head_gate: null pointer");
+  if (head_stride <= 0 || ldx < n_heads * head_stride || ldg < n_heads)
+    FAIL("head_gate: %d heads of %d columns in rows of %d, gates in rows of %d", n_heads, head_stride, ldx, ldg);
+  if (dtype != DT_F32 && dtype != DT_BF16) FAIL("head_gate: unknown dtype code %d", dtype);
+  const long total = (long)n_rows * n_heads * head_stride;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(head_gate_kernel<float>, grid, block, 0, stream, (float*)x, ldx, head_stride, n_heads, g, ldg, n_rows);
+  else
+    hipLaunchKernelGGL(head_gate_kernel<bf16>, grid, block, 0, stream, (bf16*)x, ldx, head_stride, n_heads, g, ldg, n_rows);
+  CHECK_LAUNCH("head_gate");
+  return 0;
+}

@@ -51,7 +51,18 @@ struct ScanArgs {
   const int* slot_ids;
   int n_requests, H, Hk, N, P;
   int n_tokens_hint;  // the token rows of q and k (the kernels that take chunks turn them all at once, in place)
+  // A decay per key channel instead of one a head: chan_a [tokens, ldca], head h at column h * N,
+  // holds log a (<= 0), or, with chan_logit, a logit z with log a = chan_mult * log sigmoid(z).
+  const float* chan_a;
+  int ldca, chan_logit;
+  float chan_mult;
+  const float* norm_w;  // [P] or null: with unit_rms, the normed output times this weight
 };
+
+__device__ __forceinline__ float channel_log_decay(const ScanArgs& a, size_t row, int h, int i) {
+  const float z = a.chan_a[row * a.ldca + (size_t)h * a.N + i];
+  return a.chan_logit ? -a.chan_mult * softplus_f(-z) : z;
+}
 
 // One block a (head, request); the state in LDS as S[i * P + p], thread (part, p) walks its share
 // of the keys i for value column p.  Tokens in turn: the recurrence as written.
@@ -67,6 +78,7 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
   float* ks = qs + N;
   float* vs = ks + N;
   float* partial = vs + P;  // [parts, P]
+  float* as = partial + (size_t)parts * P;  // [N], where every key channel has a decay of its own
   const int start = a.seq_start[r], n = a.seq_len[r];
   float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P;
   for (int base = 0; base < N * P; base += 256 * 8) {  // (eight loads a thread on their way at once)
@@ -99,15 +111,16 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
           qv = qr[j + half] * cs + qr[j] * sn, kv = kr[j + half] * cs + kr[j] * sn;
       }
       qs[i] = qv, ks[i] = kv * ksc;
+      if (a.chan_a) as[i] = expf(channel_log_decay(a, row, h, i));
     }
     for (int c = tid; c < P; c += 256) vs[c] = a.v[row * a.ldv + (size_t)h * P + c];
-    const float at = a.log_a ? expf(a.log_a[row * a.H + h]) : a.decay[h];
+    const float at = a.chan_a ? 1.f : a.log_a ? expf(a.log_a[row * a.H + h]) : a.decay[h];
     __syncthreads();
     if (works) {
       const float vp = vs[p];
       float acc = 0.f;
       for (int i = i0; i < i1; ++i) {
-        const float s = at * S[(size_t)i * P + p] + ks[i] * vp;
+        const float s = (a.chan_a ? as[i] : at) * S[(size_t)i * P + p] + ks[i] * vp;
         S[(size_t)i * P + p] = s;
         acc += s * qs[i];
       }
@@ -122,6 +135,7 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
     if (a.unit_rms) {
       const float ss = block_sum(tid < P ? o * o : 0.f, red);
       o *= 1.0f / sqrtf(ss / (float)P + a.eps);
+      if (a.norm_w && tid < P) o *= a.norm_w[tid];
     }
     if (tid < P) {
       if (a.gate) o *= silu_f(a.gate[row * a.ldg + (size_t)h * P + tid]);
@@ -507,14 +521,15 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
     FAIL("state_scan: null pointer");
   if (a.N <= 0 || a.P <= 0 || a.P > 256) FAIL("state_scan: key size %d, value size %d (at most 256)", a.N, a.P);
   if (a.Hk <= 0 || a.H % a.Hk) FAIL("state_scan: %d heads over %d key heads", a.H, a.Hk);
-  if (!a.log_a && !a.decay) FAIL("state_scan: a decay per token or per head is needed");
+  if (!a.log_a && !a.decay && !a.chan_a) FAIL("state_scan: a decay per token, per head or per key channel is needed");
+  if (a.chan_a && (a.ldca < a.H * a.N || a.Hk != a.H)) FAIL("state_scan: decays per key channel come in rows of heads x keys");
   if (a.rot_dims && (a.rot_dims % 2 || a.rot_dims > a.N || !a.inv_freq || !a.positions))
     FAIL("state_scan: %d turning columns of %d", a.rot_dims, a.N);
   if (a.ldq < a.Hk * a.N || a.ldk < a.Hk * a.N || a.ldv < a.H * a.P || a.ldo < a.H * a.P || (a.gate && a.ldg < a.H * a.P))
     FAIL("state_scan: a row is narrower than its heads");
   if (a.out_dtype != DT_F32 && a.out_dtype != DT_BF16) FAIL("state_scan: unknown dtype code %d", a.out_dtype);
   const int parts = a.N < 256 / a.P ? a.N : 256 / a.P;
-  const size_t lds = ((size_t)a.N * a.P + 2 * (size_t)a.N + a.P + (size_t)parts * a.P) * sizeof(float);
+  const size_t lds = ((size_t)a.N * a.P + 3 * (size_t)a.N + a.P + (size_t)parts * a.P) * sizeof(float);
   if (lds > SCAN_MAX_LDS) FAIL("state_scan: a state of %d x %d does not fit a block's LDS", a.N, a.P);
   static bool raised = false;
   if (!raised) {
@@ -524,7 +539,7 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
   }
   dim3 grid(a.H, a.n_requests), block(256);
   int C = 0;
-  if (chunked)
+  if (chunked && !a.chan_a)  // (decays per key channel: token by token)
     for (int c = 64; c >= 16 && !C; c /= 2)
       if (chunk_floats(a.N, a.P, c) * sizeof(float) <= SCAN_MAX_LDS) C = c;
   if (C) {

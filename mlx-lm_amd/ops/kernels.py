@@ -882,7 +882,8 @@ class ScanArgs(ctypes.Structure):
                 ("gate", _vp), ("ldg", _c_int), ("out", _vp), ("ldo", _c_int), ("out_dtype", _c_int),
                 ("state", _vp), ("state_stride", _c_size_t), ("state_offset", _c_size_t), ("seq_start", _vp),
                 ("seq_len", _vp), ("slot_ids", _vp), ("n_requests", _c_int), ("H", _c_int), ("Hk", _c_int),
-                ("N", _c_int), ("P", _c_int), ("n_tokens_hint", _c_int)]
+                ("N", _c_int), ("P", _c_int), ("n_tokens_hint", _c_int), ("chan_a", _vp), ("ldca", _c_int),
+                ("chan_logit", _c_int), ("chan_mult", _c_float), ("norm_w", _vp)]
 
 
 def _f32_rows(t, name, min_cols):
@@ -894,7 +895,8 @@ def _f32_rows(t, name, min_cols):
 
 def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, n_requests, n_heads, n_key_heads,
                key_dim, value_dim, log_a=None, decay=None, k_scale=None, k_mult=1.0, skip=None, rot_dims=0,
-               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None, chunked=False, spans=None):
+               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None, chunked=False, spans=None,
+               channel_decay=None, channel_logit_mult=None, norm_weight=None):
     """``S = a S + k v^T; o = S^T q`` token by token for every (request, head), from and into the
     requests' rows of ``state`` (float32 ``[slots, floats a request]``, head ``h``'s matrix
     ``[key_dim, value_dim]`` at ``state_offset + h * key_dim * value_dim``).  ``q``, ``k``
@@ -907,6 +909,10 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
     span_first, alloc)`` cuts long portions into spans that run side by side (int32 device arrays:
     the request and the first token of every span, counted from the request's first token of
     this step, and every request's first span; ``alloc(shape, dtype)`` gives the work memory).
+    ``channel_decay`` (float32 ``[tokens, >= n_heads * key_dim]``): a decay for every key channel
+    instead of one a head, given as its logarithm, or, with ``channel_logit_mult = m``, as a logit
+    ``z`` with ``log a = m * log sigmoid(z)``.  ``norm_weight`` (float32 ``[value_dim]``): with
+    ``unit_rms``, the normed output times this weight, the same for every head.
     See csrc/linear_state.hip for the options."""
     lib = build.load("linear_state")
     a = ScanArgs()
@@ -925,7 +931,18 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
             _dev(t, name, torch.float32)
             _need(t.numel() == n_heads, f"state_scan: {name} has one value a head")
             setattr(a, name, t.data_ptr())
-    _need(log_a is not None or decay is not None, "state_scan: a decay per token or per head is needed")
+    _need(log_a is not None or decay is not None or channel_decay is not None,
+          "state_scan: a decay per token, per head or per key channel is needed")
+    if channel_decay is not None:
+        _need(n_key_heads == n_heads, "state_scan: decays per key channel need a key head for every head")
+        a.ldca, a.chan_a = _f32_rows(channel_decay, "channel_decay", n_heads * key_dim), channel_decay.data_ptr()
+        _need(channel_decay.shape[0] >= T, "state_scan: fewer decay rows than output rows")
+        if channel_logit_mult is not None:
+            a.chan_logit, a.chan_mult = 1, float(channel_logit_mult)
+    if norm_weight is not None:
+        _dev(norm_weight, "norm_weight", torch.float32)
+        _need(unit_rms and norm_weight.numel() == value_dim, "state_scan: norm_weight has value_dim values and goes with unit_rms")
+        a.norm_w = norm_weight.data_ptr()
     a.k_mult = float(k_mult)
     if rot_dims:
         _dev(inv_freq, "inv_freq", torch.float32)
@@ -960,6 +977,131 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
         rc = lib.state_scan(ctypes.byref(a), _c_int(int(bool(chunked))), _c_int(0), _c_int(0), None, None, None, None, None,
                             _stream())
     build.check(lib, rc, "state_scan")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# between a projection and the attention that reads its heads, and behind it (csrc/head_prepare.hip)
+
+
+def causal_conv(y, u, col, weight, bias, state, conv_offset, token_req, seq_start, slot_ids, silu=False, single_tokens=False):
+    """``y[t, c] = act(bias[c] + sum_j weight[c, j] * u[t - taps + 1 + j, col + c])`` over each request's own
+    tokens; the inputs of earlier steps come from the request's row of ``state`` (``[taps - 1,
+    channels]`` at ``conv_offset``, the latest last; ``conv_state_update`` brings it up to date
+    afterwards, or this kernel itself with ``single_tokens``, when every request brings one token).
+    ``u`` and ``y`` are float32 rows."""
+    lib = build.load("head_prepare")
+    C, taps = weight.shape
+    ldu, ldy = _f32_rows(u, "u", col + C), _f32_rows(y, "y", C)
+    _dev(weight, "weight", torch.float32)
+    _dev(state, "state", torch.float32)
+    _need(weight.is_contiguous() and (bias is None or bias.numel() == C), "causal_conv: weight [channels, taps], bias [channels]")
+    _need(state.dim() == 2 and conv_offset + (taps - 1) * C <= state.shape[1], "causal_conv: the state rows are too short")
+    for name, t in (("token_req", token_req), ("seq_start", seq_start), ("slot_ids", slot_ids)):
+        _dev(t, name, torch.int32)
+    T = y.shape[0]
+    _need(u.shape[0] >= T and token_req.numel() >= T, "causal_conv: fewer input rows than output rows")
+    rc = lib.causal_conv(_ptr(u), _c_int(ldu), _c_int(col), _ptr(weight), _ptr(bias), _c_int(taps), _c_int(C),
+                         _c_int(int(bool(silu))), _ptr(state), _c_size_t(state.stride(0)), _c_size_t(conv_offset),
+                         _ptr(token_req), _ptr(seq_start), _ptr(slot_ids), _ptr(y), _c_int(ldy), _c_int(T),
+                         _c_int(int(bool(single_tokens))), _stream())
+    build.check(lib, rc, "causal_conv")
+    return y
+
+
+class PrepareArgs(ctypes.Structure):
+    """Mirror of ``PrepareArgs`` in csrc/head_prepare.hip."""
+
+    _fields_ = [("src", _vp), ("lds", _c_int), ("src_col", _c_int), ("src_stride", _c_int), ("n_rows", _c_int),
+                ("n_heads", _c_int), ("dim", _c_int), ("norm_dim", _c_int), ("norm_w", _vp), ("eps", _c_float),
+                ("rot_off", _c_int), ("rot_dims", _c_int), ("interleaved", _c_int), ("inv_freq", _vp),
+                ("rot_mult", _c_float), ("positions", _vp), ("dst", _vp), ("ldd", _c_int), ("dst_stride", _c_int),
+                ("dst_fill", _c_int), ("copies", _c_int), ("dst_head", _vp)]
+
+
+def head_prepare(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=None, dst_fill=None, norm_dim=0,
+                 norm_weight=None, eps=0.0, rot_off=0, rot_dims=0, inv_freq=None, rot_mult=1.0, interleaved=True,
+                 positions=None, dst_head=None, copies=1):
+    """Heads of a float32 projection row on their way to an attention: head ``h`` is ``dim`` columns
+    of ``src`` from ``src_col + h * src_stride``; RMS norm over its first ``norm_dim`` columns
+    (times ``norm_weight``, shared by the heads); rotation of ``rot_dims`` columns from ``rot_off``
+    by ``position * inv_freq[i]`` (pairs ``(2i, 2i + 1)`` with ``interleaved``, else ``(i, i +
+    rot_dims / 2)``; cos and sin times ``rot_mult``); written to ``dst`` (float32 or bfloat16) at
+    column ``dst_head[c, h] * dst_stride`` for each of ``copies`` copies (``h * dst_stride`` without
+    a table), with zeros from ``dim`` up to ``dst_fill`` columns."""
+    lib = build.load("head_prepare")
+    a = PrepareArgs()
+    src_stride = dim if src_stride is None else src_stride
+    dst_stride = dim if dst_stride is None else dst_stride
+    a.lds = _f32_rows(src, "src", src_col + (n_heads - 1) * src_stride + dim)
+    a.src, a.src_col, a.src_stride = src.data_ptr(), int(src_col), int(src_stride)
+    a.n_rows, a.n_heads, a.dim = dst.shape[0], int(n_heads), int(dim)
+    _need(src.shape[0] >= dst.shape[0], "head_prepare: fewer source rows than rows of dst")
+    a.norm_dim, a.eps = int(norm_dim), float(eps)
+    if norm_weight is not None:
+        _dev(norm_weight, "norm_weight", torch.float32)
+        _need(norm_weight.numel() == norm_dim, "head_prepare: norm_weight has norm_dim values")
+        a.norm_w = norm_weight.data_ptr()
+    if rot_dims:
+        _dev(inv_freq, "inv_freq", torch.float32)
+        _dev(positions, "positions", torch.int32)
+        _need(inv_freq.numel() == rot_dims // 2 and positions.numel() >= dst.shape[0], "head_prepare: inv_freq / positions")
+        a.rot_off, a.rot_dims, a.interleaved = int(rot_off), int(rot_dims), int(bool(interleaved))
+        a.inv_freq, a.rot_mult, a.positions = inv_freq.data_ptr(), float(rot_mult), positions.data_ptr()
+    a.ldd = _rows2d(dst, "dst")
+    _need(dst.dtype in DT, "head_prepare: dst is float32 or bfloat16")
+    a.dst, a.dst_stride, a.dst_fill, a.copies = dst.data_ptr(), int(dst_stride), int(dst_fill or dim), int(copies)
+    if dst_head is not None:
+        _dev(dst_head, "dst_head", torch.int32)
+        _need(dst_head.numel() == copies * n_heads, "head_prepare: dst_head is [copies, heads]")
+        a.dst_head = dst_head.data_ptr()
+    _need(dst.shape[1] >= (n_heads * copies - 1) * dst_stride + a.dst_fill, "head_prepare: dst rows are too short for the heads")
+    rc = lib.head_prepare(ctypes.byref(a), _c_int(DT[dst.dtype]), _stream())
+    build.check(lib, rc, "head_prepare")
+    return dst
+
+
+def diff_combine(out, att, head_stride, first, second, lam, mult, eps, vdim):
+    """``out[t, h] = mult * unit_rms(att[t, first[h]] - lam * att[t, second[h]])`` over the first
+    ``vdim`` columns of heads that lie ``head_stride`` apart in ``att``."""
+    lib = build.load("head_prepare")
+    lda, ldo = _rows2d(att, "att"), _rows2d(out, "out")
+    _dev(first, "first", torch.int32)
+    _dev(second, "second", torch.int32)
+    n_heads = first.numel()
+    _need(second.numel() == n_heads and out.dtype == att.dtype and att.dtype in DT and att.shape[0] >= out.shape[0], "diff_combine: shapes")
+    rc = lib.diff_combine(_ptr(att), _c_int(lda), _c_int(head_stride), _ptr(first), _ptr(second), _c_float(lam), _c_float(mult),
+                          _c_float(eps), _c_int(out.shape[0]), _c_int(n_heads), _c_int(vdim), _ptr(out), _c_int(ldo),
+                          _c_int(DT[out.dtype]), _stream())
+    build.check(lib, rc, "diff_combine")
+    return out
+
+
+def head_gate(x, head_stride, n_heads, gate):
+    """``x[t, h, :] *= sigmoid(gate[t, h])`` in place; ``gate`` float32 rows of at least ``n_heads`` columns."""
+    lib = build.load("head_prepare")
+    ldx, ldg = _rows2d(x, "x"), _f32_rows(gate, "gate", n_heads)
+    _need(x.dtype in DT and x.shape[1] >= n_heads * head_stride and gate.shape[0] >= x.shape[0], "head_gate: shapes")
+    rc = lib.head_gate(_ptr(x), _c_int(ldx), _c_int(head_stride), _c_int(n_heads), _ptr(gate), _c_int(ldg),
+                       _c_int(x.shape[0]), _c_int(DT[x.dtype]), _stream())
+    build.check(lib, rc, "head_gate")
+    return x
+
+
+def attend(ctx, out, q, cache, n_heads, n_kv_heads, head_dim, scale, window=0):
+    """Causal attention of the step's queries ``q`` ``[tokens, n_heads * head_dim]`` over the pages
+    of ``cache`` (a ``CacheView``), into ``out``: the native host chooses among the attention kernels
+    as it does for the built-in attention part (single rows to the decode kernels, portions to the
+    tile kernels), by the step arrays that part declares (``parts.attention.CausalSelfAttention``:
+    a mixer that calls this names the same ``step_arrays_key``)."""
+    from ..parts.attention import CausalSelfAttention as A
+
+    base = native.array_ids(A.step_arrays_key, A.step_array_names)
+    qm, om = native.mat(q), native.mat(out)
+    with ctx.enter():
+        rc = native.lib().eng_attend(ctypes.byref(ctx.c), ctypes.byref(om), ctypes.byref(qm), cache.slot, int(n_heads),
+                                     int(n_kv_heads), int(head_dim), int(window), float(scale), base)
+    native.check(rc, "attend")
     return out
 
 

@@ -26,7 +26,7 @@ TORCH_DT = {0: torch.float32, 1: torch.bfloat16, 2: torch.int32}
 # kinds of part and callback methods (csrc/engine.h)
 NORM, MIXER, FFN, BLOCK, POSITION, EMBEDDING, HEAD, MODEL = range(1, 9)
 CB_NORM, CB_MIXER, CB_FFN, CB_BLOCK, CB_ROTATE, CB_EMBEDDING_TERM, CB_EMBEDDING, CB_HEAD, CB_GROW = range(1, 10)
-ACCEPTS_LAZY, SETTLES_PENDING, HANDLES_PENDING, READS_AHEAD = 1, 2, 4, 8
+ACCEPTS_LAZY, SETTLES_PENDING, HANDLES_PENDING, READS_AHEAD, WANTS_STATE = 1, 2, 4, 8, 16
 
 
 class EngMat(Structure):
@@ -165,6 +165,8 @@ def lib():
                                      POINTER(EngValue)]),
         "eng_mixer_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngValue), POINTER(EngMat), c_int, c_int]),
         "eng_ffn_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngValue), POINTER(EngMat)]),
+        "eng_attend": (c_int, [POINTER(EngCtx), POINTER(EngMat), POINTER(EngMat), c_int, c_int, c_int, c_int, c_int,
+                               c_float, c_int]),
         "eng_embedding_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngMat), P]),
         "eng_head_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngValue), POINTER(EngMat)]),
         "eng_settle": (c_int, [POINTER(EngCtx)]),
@@ -297,7 +299,11 @@ def run_python_part(part, method, ctx, call):
     """A callback part's turn: build tensors over the native side's matrices, call the method."""
     T = ctx.tensor
     if method == CB_MIXER:
-        part.forward(ctx, T(call.x), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache))
+        if call.state_slot >= 0 and getattr(part, "wants_state", False):
+            part.forward(ctx, T(call.x), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache),
+                         state=ctx.cache_view(call.state_slot))
+        else:
+            part.forward(ctx, T(call.x), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache))
     elif method == CB_FFN:
         part.forward(ctx, T(call.x), T(call.residual))
     elif method == CB_BLOCK:

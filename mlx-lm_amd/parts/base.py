@@ -77,6 +77,8 @@ class Part:
         flags = 0
         if getattr(self, "settles_pending", False):
             flags |= native.SETTLES_PENDING
+        if getattr(self, "wants_state", False):
+            flags |= native.WANTS_STATE
         self._python_id = native.register_python_part(self)
         return native.made(native.lib().eng_make_callback(self.native_kind, self._python_id, flags),
                            type(self).__name__)

@@ -17,31 +17,53 @@ class PreNormBlock(Block):
     idle may have them read the weights that come after its own (the
     feed-forward's first).  The arrangement itself runs in the native host
     (``PreNormBlock`` in csrc/engine.hip); its parts may be native or Python.
+    The feed-forward, with its norm, may be absent.  A mixer that keeps per-request state beside
+    its pages (``wants_state`` and ``state_need()``) gets the run's state slot too.
     """
 
     PARTS = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
+    OPTIONAL = ("ffn_norm", "ffn")
     handles_pending = True
 
-    def __init__(self, mixer_norm, mixer, ffn_norm, ffn, prefix=""):
+    def __init__(self, mixer_norm, mixer, ffn_norm=None, ffn=None, prefix=""):
         super().__init__(prefix)
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a pre-norm layer has a feed-forward and its norm, or neither")
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.parts())
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        out = []
+
+        def walk(part):
+            if part is None:
+                return
+            out.append(part)
+            for sub in getattr(part, "sub_parts", lambda: ())():
+                walk(sub)
+
+        for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn):
+            walk(p)
+        return tuple(out)
 
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def state_need(self):
+        if getattr(self.mixer, "wants_state", False) and hasattr(self.mixer, "state_need"):
+            return self.mixer.state_need()
+        return None
+
     def make_native(self):
         return native.made(native.lib().eng_make_pre_norm_block(
-            self.mixer_norm.native(), self.mixer.native(), self.ffn_norm.native(), self.ffn.native()),
-            "pre-norm block")
+            self.mixer_norm.native(), self.mixer.native(), self.ffn_norm.native() if self.ffn_norm is not None else None,
+            self.ffn.native() if self.ffn is not None else None), "pre-norm block")
 
-    def forward(self, ctx, h, cache, writes_cache=True):
+    def forward(self, ctx, h, cache, writes_cache=True, state=None):
         hm = native.mat(h)
         with ctx.enter():
             rc = native.lib().eng_block_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(hm), cache.slot,
-                                                int(bool(writes_cache)), -1)
+                                                int(bool(writes_cache)), state.slot if state is not None else -1)
         native.check(rc, "pre-norm block")
         return h
 

@@ -1,0 +1,52 @@
+"""A short causal convolution over time on each channel of a projection's output."""
+
+from ..config.plan import StateNeed
+from ..ops import kernels
+from .base import Part, TensorSpec
+from .linear_state import _SequenceArrays
+
+
+class ShortConvolution(_SequenceArrays, Part):
+    """``y_t = sum_j w[:, j] * u_(t - taps + 1 + j)`` per channel, zeros before a request's first
+    token, no bias.  The channels of several tensors (``names``: a tensor ``[channels, taps]``
+    each) lie side by side in one row.  The last ``taps - 1`` inputs of a request are its state,
+    kept in the request's row of a state slot that the mixer which owns this part asks for
+    (``state_need``) and zeroed when a request starts, which gives the zeros before its first token.
+    Not a mixer: a mixer builds it, runs it between its projection and what follows, and lists it
+    among its ``sub_parts`` so that the model hands it its tensors and its step arrays (where each
+    request's tokens start).  32-bit throughout (csrc/head_prepare.hip: ``causal_conv``).  No
+    counterpart in mlx_lm/models/gpt2.py."""
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, channels, taps, names, prefix=""):
+        super().__init__(prefix)
+        if taps < 1 or not channels or any(c <= 0 for c in channels) or len(channels) != len(names):
+            raise ValueError(f"{taps} taps over channels {channels} of tensors {names}")
+        self.channels, self.taps = [int(c) for c in channels], int(taps)
+        self.n_channels = sum(self.channels)
+        self.names = [self._name(n) for n in names]
+        self.state_floats = (self.taps - 1) * self.n_channels
+        self.weight = None
+
+    def tensors(self):
+        return {n: TensorSpec((c, self.taps), "vector") for n, c in zip(self.names, self.channels)}
+
+    def load(self, tensors):
+        import torch
+
+        self.weight = torch.cat([tensors[n] for n in self.names]).contiguous()
+
+    def state_need(self):
+        return StateNeed((self.state_floats,), "float32") if self.state_floats else None
+
+    def forward(self, ctx, y, u, state, offset=0):
+        """``y`` from ``u`` (float32 rows of ``n_channels`` columns from column 0); ``state``: the
+        requests' state rows, this part's floats from ``offset`` on."""
+        starts = ctx.array("sequences.starts")
+        single = ctx.array("sequences.longest") == 1
+        kernels.causal_conv(y, u, 0, self.weight, None, state, offset, ctx.token_req, starts, ctx.slot_ids,
+                            single_tokens=single)
+        if not single and self.taps > 1:
+            kernels.conv_state_update(u, 0, self.taps, self.n_channels, state, offset, starts, ctx.array("sequences.lens"),
+                                      ctx.slot_ids, ctx.n_requests)

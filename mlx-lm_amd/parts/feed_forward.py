@@ -118,5 +118,54 @@ class Relu2MLP(FeedForward):
         native.check(rc, "relu2_mlp")
 
 
+class GatedMLP(FeedForward):
+    """``down(silu(gate(x)) * up(x))``, dense, no biases.
+
+    One product gives ``[gate | up]``; the activation and the product of the two halves are one
+    kernel (``silu_mul``, which the experts' shared expert uses too); the second product adds into
+    ``residual``.  No counterpart in mlx_lm/models/gpt2.py, whose MLP (:71-80) has no gate.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, width, inner, gate_name="gate", up_name="up", down_name="down", prefix=""):
+        super().__init__(prefix)
+        if width % 8:
+            raise ValueError(f"the feed-forward's width must be a multiple of 8, got {width}")
+        if inner <= 0:
+            raise ValueError(f"the feed-forward's inner size must be positive, got {inner}")
+        self.width, self.inner = width, inner
+        self.inner_padded = (inner + 7) // 8 * 8  # zero weights beyond ``inner``: silu(0) * 0 = 0 meets zero columns
+        self.gate_name, self.up_name, self.down_name = self._name(gate_name), self._name(up_name), self._name(down_name)
+        self.gate_up_w = self.down_w = None
+
+    def tensors(self):
+        return {self.gate_name: TensorSpec((self.inner, self.width), "matrix"),
+                self.up_name: TensorSpec((self.inner, self.width), "matrix"),
+                self.down_name: TensorSpec((self.width, self.inner), "matrix")}
+
+    def load(self, tensors):
+        gate, up, down = tensors[self.gate_name], tensors[self.up_name], tensors[self.down_name]
+        pad = self.inner_padded - self.inner
+        if pad:
+            zeros = gate.new_zeros(pad, self.width)
+            gate, up = torch.cat([gate, zeros]), torch.cat([up, zeros])
+            down = torch.cat([down, down.new_zeros(self.width, pad)], dim=1)
+        self.gate_up_w = kernels.for_decode(torch.cat([gate, up]).contiguous())
+        self.down_w = kernels.for_decode(down.contiguous())
+        self.first_weight = self.gate_up_w
+
+    def forward(self, ctx, x, residual):
+        T, F = x.shape[0], self.inner_padded
+        mark = ctx.scratch_mark()
+        gate_up = ctx.scratch((T, 2 * F), ctx.dtype)
+        kernels.linear(gate_up, x, self.gate_up_w, splits=kernels.splits_alone(T))
+        act = ctx.scratch((T, F), ctx.dtype)
+        kernels.silu_mul(act, gate_up)
+        kernels.linear(residual, act, self.down_w, accumulate=True, splits=kernels.splits_alone(T))
+        ctx.scratch_release(mark)
+
+
 register_feed_forward("gelu_mlp", GeluMLP)
+register_feed_forward("gated_mlp", GatedMLP)
 register_feed_forward("relu2_mlp", Relu2MLP)

@@ -138,6 +138,83 @@ class Retention(_SequenceArrays, Mixer):
         ctx.scratch_release(mark)
 
 
+class GatedLinearAttention(_SequenceArrays, Mixer):
+    """Linear attention whose state decays by a gate of its own for every key channel:
+
+        ``S_t = diag(alpha_t) S_(t-1) + k_t v_t^T``,   ``o_t = S_t^T q_t``
+
+    with ``q = Wq x * key_dim^(-1/2)``, ``k = Wk x`` (``n_heads x key_dim``), ``v = Wv x`` (``n_heads x
+    value_dim``) and ``alpha = sigmoid(z)^(1 / tau)``, ``z = Wa2 (Wa1 x) + b`` through a narrow
+    middle, laid out like the keys.  Each head's ``o`` is RMS-normed over ``value_dim`` with one
+    weight for all heads, the heads are multiplied by ``silu(Wg x)`` and projected by ``Wo``.
+    ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start) is the request's
+    state.  One product gives ``[q | k | v | g]`` as float32 rows; ``z`` is a float32 row; the
+    logarithm of the decay (``log sigmoid(z) / tau``), the recurrence, the norm and the gate are
+    32-bit (csrc/linear_state.hip; the factor of the queries rides on the keys, which gives the
+    same outputs).  No counterpart in mlx_lm/models/gpt2.py.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, width, n_heads, key_dim, value_dim, tau, eps, decay_rank, prefix=""):
+        super().__init__(prefix)
+        if n_heads <= 0 or key_dim <= 0 or not 0 < value_dim <= 256 or decay_rank <= 0:
+            raise ValueError(f"{n_heads} heads of keys {key_dim} and values {value_dim} (values at most 256), a middle of {decay_rank}")
+        if tau <= 0:
+            raise ValueError(f"tau must be positive, got {tau}")
+        if width % 8:
+            raise ValueError(f"width {width} must be a multiple of 8")
+        self.width, self.n_heads, self.key_dim, self.value_dim = width, n_heads, key_dim, value_dim
+        self.tau, self.eps, self.decay_rank = float(tau), float(eps), int(decay_rank)
+        self.qk_width, self.v_width = n_heads * key_dim, n_heads * value_dim
+
+    def cache_need(self):
+        return StateNeed((self.n_heads * self.key_dim * self.value_dim,), "float32")
+
+    def tensors(self):
+        n = self._name
+        return {n("q"): TensorSpec((self.qk_width, self.width), "matrix"),
+                n("k"): TensorSpec((self.qk_width, self.width), "matrix"),
+                n("v"): TensorSpec((self.v_width, self.width), "matrix"),
+                n("g"): TensorSpec((self.v_width, self.width), "matrix"),
+                n("o"): TensorSpec((self.width, self.v_width), "matrix"),
+                n("norm"): TensorSpec((self.value_dim,), "vector"),
+                n("a1"): TensorSpec((self.decay_rank, self.width), "matrix"),
+                n("a2"): TensorSpec((self.qk_width, self.decay_rank), "matrix"),
+                n("a2.b"): TensorSpec((self.qk_width,), "vector")}
+
+    def load(self, tensors):
+        n = self._name
+        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in ("q", "k", "v", "g")]))
+        self.first_weight = self.in_w
+        a1 = tensors[n("a1")]
+        pad = -a1.shape[0] % 8  # (the middle is the second product's inner size: zero rows here meet zero columns there)
+        self.a1_w = _matrix(torch.cat([a1, a1.new_zeros(pad, a1.shape[1])]) if pad else a1)
+        self.a2_w, self.a2_b = _matrix(_padded_columns(tensors[n("a2")])), tensors[n("a2.b")]
+        self.out_w = _matrix(_padded_columns(tensors[n("o")]))
+        self.norm_w = tensors[n("norm")]
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True):
+        T = x.shape[0]
+        mark = ctx.scratch_mark()
+        u = ctx.scratch((T, 2 * self.qk_width + 2 * self.v_width), torch.float32)
+        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
+        mid = ctx.scratch((T, -(-self.decay_rank // 8) * 8), ctx.dtype)
+        kernels.linear(mid, x, self.a1_w, splits=kernels.splits_alone(T))
+        z = ctx.scratch((T, self.qk_width), torch.float32)
+        kernels.linear(z, mid, self.a2_w, bias=self.a2_b, splits=kernels.splits_alone(T))
+        a, b = self.qk_width, 2 * self.qk_width
+        out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
+        kernels.state_scan(out, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, 0,
+                           ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,
+                           self.n_heads, self.n_heads, self.key_dim, self.value_dim, channel_decay=z,
+                           channel_logit_mult=1.0 / self.tau, k_mult=self.key_dim**-0.5, unit_rms=True, eps=self.eps,
+                           norm_weight=self.norm_w, gate=u[:, b + self.v_width:], chunked=self._chunked(ctx),
+                           spans=self._spans(ctx))
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=True, splits=kernels.splits_alone(T))
+        ctx.scratch_release(mark)
+
+
 class StateSpace(_SequenceArrays, Mixer):
     """The selective state space with a scalar decay a head:
 
@@ -278,5 +355,6 @@ class ParallelMixers(Mixer):
 
 
 register_mixer("retention", Retention)
+register_mixer("gated_linear_attention", GatedLinearAttention)
 register_mixer("state_space", StateSpace)
 register_mixer("parallel", ParallelMixers)

@@ -54,6 +54,9 @@ def model_from_tensors(config, weights, dtype="bfloat16", device="cuda:0",
     What ``load_model`` does after reading the folder; callers that make their weights
     themselves (a benchmark's random ones) come in here."""
     model_cls, args_cls = get_model_classes(config)
+    if hasattr(args_cls, "sizes_from_tensors"):
+        # (a design may leave a size to the checkpoint: the shape of a tensor says it)
+        config = args_cls.sizes_from_tensors(config, {name: tuple(t.shape) for name, t in weights.items()})
     args = args_cls.from_dict(config)
     model = model_cls(args)
     if hasattr(model, "sanitize"):
