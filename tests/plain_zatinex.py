@@ -179,3 +179,63 @@ def forward(config, w, tokens, return_layers=False):
         streams.append(x)
     logits = rms_norm(x, w["final.norm"], eps) @ w["head"].t()
     return (logits, torch.stack(streams)) if return_layers else logits
+
+
+def random_weights(config, seed, sharp=1.0, decay_rank=4):
+    """Float32 tensors under the checkpoint's names, every vector drawn.  ``sharp`` widens the
+    attention scores (the weights of the query norms and the queries' up-projection grow by it),
+    so that a key which is dropped, doubled or taken from a wrong page shows in the logits."""
+    g = torch.Generator().manual_seed(seed)
+    D = config["width"]
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return torch.randn(*shape, generator=g) * std + mean
+
+    w = {"embed": rnd(config["vocab"], D), "final.norm": rnd(D, std=0.1, mean=1.0), "head": rnd(config["vocab"], D, std=D ** -0.5)}
+    for i, layer in enumerate(config["layers"]):
+        p, m = f"l{i}.mix.", layer["mixer"]
+        w[f"l{i}.norm1"] = rnd(D, std=0.1, mean=1.0)
+        if layer["type"] == "attention":
+            H, G, d, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
+            for name, n in (("q", 2 * H * d), ("k", 2 * G * d), ("v", G * dv)):
+                w[p + name], w[p + name + ".b"] = rnd(n, D, std=D ** -0.5), rnd(n, std=0.2)
+                if m.get("conv"):
+                    w[p + name + ".conv"] = rnd(n, m["conv"], std=0.6)
+            w[p + "q.norm"], w[p + "k.norm"] = rnd(d, std=0.2, mean=1.0) * sharp, rnd(d, std=0.2, mean=1.0)
+            for name in ("lq1", "lk1", "lq2", "lk2"):
+                w[p + name] = rnd(d, std=0.15)
+            w[p + "o"] = rnd(D, H * dv, std=(H * dv) ** -0.5)
+        elif layer["type"] == "gla":
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            for name, n in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv)):
+                w[p + name] = rnd(n, D, std=D ** -0.5)
+            w[p + "o"], w[p + "norm"] = rnd(D, H * dv, std=(H * dv) ** -0.5), rnd(dv, std=0.2, mean=1.0)
+            w[p + "a1"], w[p + "a2"] = rnd(decay_rank, D, std=D ** -0.5), rnd(H * d, decay_rank, std=1.0)
+            w[p + "a2.b"] = rnd(H * d, std=1.0, mean=1.5)
+        else:
+            H, d, dr, dv, Q, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"]
+            w[p + "dq"], w[p + "dq.norm"] = rnd(Q, D, std=D ** -0.5), rnd(Q, std=0.2, mean=1.0)
+            w[p + "uq"] = rnd(H * (d + dr), Q, std=Q ** -0.5) * sharp
+            if "kv_from" not in m:
+                w[p + "dkv"], w[p + "dkv.norm"] = rnd(R + dr, D, std=D ** -0.5), rnd(R, std=0.2, mean=1.0)
+            w[p + "uk"], w[p + "uv"] = rnd(H * d, R, std=R ** -0.5), rnd(H * dv, R, std=R ** -0.5)
+            w[p + "g"], w[p + "o"] = rnd(H, D, std=D ** -0.5), rnd(D, H * dv, std=(H * dv) ** -0.5)
+        if layer.get("mlp") is not None:
+            F = layer["mlp"]["ff"]
+            w[f"l{i}.norm2"] = rnd(D, std=0.1, mean=1.0)
+            w[f"l{i}.mlp.gate"], w[f"l{i}.mlp.up"] = rnd(F, D, std=D ** -0.5), rnd(F, D, std=D ** -0.5)
+            w[f"l{i}.mlp.down"] = rnd(D, F, std=F ** -0.5)
+    return w
+
+
+def model(weights, config, tokens):
+    """Logits ``[T, vocab]`` in float64 from float32 (or rounded) weights."""
+    return forward(config, {k: v.double() for k, v in weights.items()}, tokens)
+
+
+def greedy(weights, config, prompt, n):
+    tokens, out = list(prompt), []
+    for _ in range(n):
+        out.append(int(model(weights, config, tokens)[-1].argmax()))
+        tokens.append(out[-1])
+    return out
