@@ -380,9 +380,245 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
   if (sp.mode == SPAN_STATES && tid == 0) sp.span_decay[(size_t)blockIdx.y * a.H + h] = expf(span_log);
 }
 
+// The same chunks where every key channel i has a decay of its own (a.chan_a): with L_t[i] the sum
+// of the channel's log decays inside the chunk,
+//   o_t  = sum_i q_t[i] exp(L_t[i]) S_0[i, :] + sum_(j <= t) A[t][j] v_j,
+//   A[t][j] = sum_i q_t[i] k_j[i] exp(L_t[i] - L_j[i]),
+//   S_C[i, :] = exp(L_C[i]) S_0[i, :] + sum_j k_j[i] exp(L_C[i] - L_j[i]) v_j
+// A does not split into a product of a factor of t and a factor of j whose exponents both stay
+// <= 0, so it is made tile by tile (16 x 16 tokens): below the diagonal both operands are taken
+// to the reference b = the last token ahead of the tile's queries, q_t exp(L_t - L_b) and
+// k_j exp(L_b - L_j) (j <= b < t: both exponents <= 0), on the matrix cores; on the diagonal every
+// pair (t, j <= t) is summed as written, four lanes a pair, each a quarter of the channels, added
+// in a fixed order.  LT [Np][C + 4] holds L; afterwards QT becomes q exp(L_t) and KT becomes
+// k exp(L_C - L_j) in place, for the products with the state and into it.
+template <typename T>
+__global__ __launch_bounds__(256) void channel_chunks_kernel(ScanArgs a, int C, SpanArgs sp) {
+  extern __shared__ float lds[];
+  __shared__ float Rs[64];
+  __shared__ unsigned char pair_t[136], pair_j[136];
+  const int N = a.N, P = a.P, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int Np = (N + 15) & ~15, Pp = (P + 15) & ~15, CP = C + 4;
+  const int h = blockIdx.x;
+  const int r = sp.mode == WHOLE ? blockIdx.y : sp.span_req[blockIdx.y];
+  float* QT = lds;
+  float* KT = QT + (size_t)Np * CP;
+  float* LT = KT + (size_t)Np * CP;
+  float* V = LT + (size_t)Np * CP;
+  float* O = V + (size_t)C * Pp;
+  float* AT = O + (size_t)C * Pp;
+  float* S = AT + (size_t)C * CP;
+  float* Lsum = S + (size_t)Np * Pp;  // [Np] the log decay of every channel over the span so far
+  const int start = a.seq_start[r];
+  const int lo = sp.mode == WHOLE ? 0 : sp.span_start[blockIdx.y];
+  const int n = sp.mode == WHOLE ? a.seq_len[r] : min(a.seq_len[r], lo + sp.span);
+  float* Sg = sp.mode == WHOLE ? a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P
+                               : sp.span_state + ((size_t)blockIdx.y * a.H + h) * N * P;
+  for (int base = 0; base < Np * Pp; base += 256 * 8) {
+    float sv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = min(base + u * 256 + tid, Np * Pp - 1), kn = min(i / Pp, N - 1), p = min(i % Pp, P - 1);
+      sv[u] = sp.mode != SPAN_STATES ? Sg[(size_t)kn * P + p] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = base + u * 256 + tid;
+      if (i < Np * Pp) S[i] = i / Pp < N && i % Pp < P ? sv[u] : 0.f;
+    }
+  }
+  for (int i = tid; i < Np; i += 256) Lsum[i] = 0.f;
+  if (tid < 136) {  // the pairs (t, j <= t) of a tile of sixteen tokens, row by row
+    int t = 0;
+    while ((t + 1) * (t + 2) / 2 <= tid) ++t;
+    pair_t[tid] = (unsigned char)t, pair_j[tid] = (unsigned char)(tid - t * (t + 1) / 2);
+  }
+  const bool outputs = sp.mode != SPAN_STATES;
+  const int ct = C / 16, pt = Pp / 16, nt = Np / 16, lr = lane & 15, lg = lane >> 4;
+  for (int c0 = lo; c0 < n; c0 += C) {
+    const int m = min(C, n - c0);
+    const size_t row0 = (size_t)(start + c0);
+    const bool gates_ahead = outputs && a.gate && P <= 64;
+    float gv[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      gv[u] = gates_ahead ? a.gate[(row0 + min(wave + 4 * u, m - 1)) * a.ldg + (size_t)h * P + min(lane, P - 1)] : 0.f;
+    {
+      const int total = C * N, v_total = C * P, most = max(total, v_total);
+      const float* qb = a.q + row0 * a.ldq + (size_t)h * N;
+      const float* kb = a.k + row0 * a.ldk + (size_t)h * N;
+      const float* ab = a.chan_a + row0 * a.ldca + (size_t)h * N;
+      const float* vb = a.v + row0 * a.ldv + (size_t)h * P;
+      bool first = true;
+      for (int base = 0; base < most; base += 256 * 16) {
+        float qv[16], kv[16], av[16], vv[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int e = base + u * 256 + tid;
+          const int eq = min(e, total - 1), t = eq / N, i = eq - t * N, tc = min(t, m - 1);
+          qv[u] = qb[(size_t)tc * a.ldq + i], kv[u] = kb[(size_t)tc * a.ldk + i], av[u] = ab[(size_t)tc * a.ldca + i];
+          const int ev = min(e, v_total - 1), tv = ev / P;
+          vv[u] = vb[(size_t)min(tv, m - 1) * a.ldv + (ev - tv * P)];
+        }
+        if (first) {
+          __syncthreads();  // the chunk before is done with every array (and S is loaded)
+          for (int e = tid; e < C * CP; e += 256) AT[e] = 0.f;
+        }
+        first = false;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int e = base + u * 256 + tid;
+          if (e < total) {
+            const int t = e / N, i = e - t * N;
+            const float la = a.chan_logit ? -a.chan_mult * softplus_f(-av[u]) : av[u];
+            QT[(size_t)i * CP + t] = t < m ? qv[u] : 0.f, KT[(size_t)i * CP + t] = t < m ? kv[u] * a.k_mult : 0.f;
+            LT[(size_t)i * CP + t] = t < m ? la : 0.f;
+          }
+          if (e < v_total) {
+            const int t = e / P;
+            V[(size_t)t * Pp + (e - t * P)] = t < m ? vv[u] : 0.f;
+          }
+        }
+      }
+      for (int e = tid; e < C * (Np - N); e += 256) {  // the padding
+        const int t = e / (Np - N), i = N + e % (Np - N);
+        QT[(size_t)i * CP + t] = 0.f, KT[(size_t)i * CP + t] = 0.f, LT[(size_t)i * CP + t] = 0.f;
+      }
+      for (int e = tid; e < C * (Pp - P); e += 256) V[(size_t)(e / (Pp - P)) * Pp + P + e % (Pp - P)] = 0.f;
+    }
+    __syncthreads();
+    for (int i = tid; i < N; i += 256) {  // a channel's running sum, token after token
+      float acc = 0.f;
+      for (int t = 0; t < C; ++t) {
+        acc += LT[(size_t)i * CP + t];
+        LT[(size_t)i * CP + t] = acc;
+      }
+      Lsum[i] += acc;
+    }
+    __syncthreads();
+    if (outputs) {
+      // the diagonal tiles: lanes 4p .. 4p + 3 share pair p, a quarter of the channels each
+      const int items = ct * 136 * 4, quarter = Np / 4, part = tid & 3;
+      for (int base = 0; base < items; base += 256) {
+        const int item = base + tid, pr = min(item, items - 1) >> 2, tile = pr / 136, pp = pr - tile * 136;
+        const int t = tile * 16 + pair_t[pp], j = tile * 16 + pair_j[pp];
+        float acc = 0.f;
+        for (int i = part * quarter; i < (part + 1) * quarter; ++i) {
+          const float* row = QT + (size_t)i * CP;
+          const float* lrow = LT + (size_t)i * CP;
+          acc += row[t] * KT[(size_t)i * CP + j] * expf(lrow[t] - lrow[j]);
+        }
+        acc += __shfl_xor(acc, 1);
+        acc += __shfl_xor(acc, 2);
+        if (item < items && part == 0) AT[(size_t)j * CP + t] = acc;
+      }
+      // the tiles below the diagonal
+      const int below = ct * (ct - 1) / 2;
+      for (int tile = wave; tile < below; tile += 4) {
+        int tt = 1;
+        while (tt * (tt + 1) / 2 <= tile) ++tt;
+        const int t0 = tt * 16, j0 = (tile - tt * (tt - 1) / 2) * 16;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < Np; i += 4) {
+          const size_t ro = (size_t)(i + lg) * CP;
+          const float ref = LT[ro + t0 - 1];
+          const float qa = QT[ro + t0 + lr] * expf(LT[ro + t0 + lr] - ref);
+          const float kb_ = KT[ro + j0 + lr] * expf(ref - LT[ro + j0 + lr]);
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa, kb_, acc, 0, 0, 0);
+        }
+        float4 o = {acc[0], acc[1], acc[2], acc[3]};
+        *(float4*)(AT + (size_t)(j0 + lr) * CP + t0 + 4 * lg) = o;
+      }
+    }
+    __syncthreads();
+    const bool state_needed = sp.mode != SPAN_OUTPUTS || c0 + C < n;
+    for (int e = tid; e < Np * C; e += 256) {
+      const int i = e / C, t = e - i * C;
+      const size_t at = (size_t)i * CP + t;
+      const float l = LT[at];
+      if (outputs) QT[at] *= expf(l);
+      if (state_needed) KT[at] *= expf(LT[(size_t)i * CP + C - 1] - l);  // (from m on the sum stands still: L_C)
+    }
+    __syncthreads();
+    // O[t][p] = sum_j AT[j][t] V[j][p] + sum_i QT[i][t] S[i][p]
+    for (int tile = wave; outputs && tile < ct * pt; tile += 4) {
+      const int t0 = (tile / pt) * 16, p0 = (tile % pt) * 16;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      const int j_end = min((m + 3) & ~3, t0 + 16);
+      for (int j = 0; j < j_end; j += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(AT[(size_t)(j + lg) * CP + t0 + lr], V[(size_t)(j + lg) * Pp + p0 + lr], acc, 0, 0, 0);
+      for (int i = 0; i < Np; i += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(QT[(size_t)(i + lg) * CP + t0 + lr], S[(size_t)(i + lg) * Pp + p0 + lr], acc, 0, 0, 0);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) O[(size_t)(t0 + 4 * lg + x) * Pp + p0 + lr] = acc[x];
+    }
+    __syncthreads();
+    // S[i][:] = exp(L_C[i]) S[i][:] + sum_j KT[i][j] V[j][:]
+    for (int tile = wave; state_needed && tile < nt * pt; tile += 4) {
+      const int i0 = (tile / pt) * 16, p0 = (tile % pt) * 16;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      const int j_end = (m + 3) & ~3;
+      for (int j = 0; j < j_end; j += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(KT[(size_t)(i0 + lr) * CP + j + lg], V[(size_t)(j + lg) * Pp + p0 + lr], acc, 0, 0, 0);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int i = i0 + 4 * lg + x;
+        float* sp_ = S + (size_t)i * Pp + p0 + lr;
+        *sp_ = expf(LT[(size_t)i * CP + C - 1]) * *sp_ + acc[x];
+      }
+    }
+    // the rows on their way out: a wave a token
+    if (outputs && a.unit_rms)
+      for (int t = wave; t < m; t += 4) {
+        float ss = 0.f;
+        for (int pc = lane; pc < P; pc += 64) ss += O[(size_t)t * Pp + pc] * O[(size_t)t * Pp + pc];
+        ss = wave_sum(ss);
+        if (lane == 0) Rs[t] = 1.0f / sqrtf(ss / (float)P + a.eps);
+      }
+    if (gates_ahead || (outputs && !a.gate && P <= 64)) {
+      const float nw = a.norm_w && a.unit_rms ? a.norm_w[min(lane, P - 1)] : 1.f;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int t = wave + 4 * u;
+        if (t >= m || lane >= P) continue;
+        float o = O[(size_t)t * Pp + lane];
+        if (a.unit_rms) o *= Rs[t] * nw;
+        if (a.gate) o *= silu_f(gv[u]);
+        ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + lane] = from_f32<T>(o);
+      }
+    } else {
+      for (int pb = 0; outputs && pb < P; pb += 64) {
+        const int pc = min(pb + lane, P - 1);
+        const float nw = a.norm_w && a.unit_rms ? a.norm_w[pc] : 1.f;
+        for (int tb = wave; tb < m; tb += 32) {
+          float g8[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            g8[u] = a.gate ? a.gate[(row0 + min(tb + 4 * u, m - 1)) * a.ldg + (size_t)h * P + pc] : 0.f;
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int t = tb + 4 * u;
+            if (t >= m || pb + lane >= P) continue;
+            float o = O[(size_t)t * Pp + pc];
+            if (a.unit_rms) o *= Rs[t] * nw;
+            if (a.gate) o *= silu_f(g8[u]);
+            ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + pc] = from_f32<T>(o);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (sp.mode == SPAN_OUTPUTS) return;
+  for (int i = tid; i < N * P; i += 256) Sg[i] = S[(size_t)(i / P) * Pp + i % P];
+  if (sp.mode == SPAN_STATES)  // (span_decay has a value for every channel here)
+    for (int i = tid; i < N; i += 256) sp.span_decay[((size_t)blockIdx.y * a.H + h) * N + i] = expf(Lsum[i]);
+}
+
 // Block (head, request, 256 elements of the state), a thread an element: span_state[s] becomes
 // the state ahead of span s, and the request's row its state after the last span.  Four spans'
-// values are asked for before the first is used.
+// values are asked for before the first is used.  With decays per key channel span_decay is
+// [spans, H, N], else [spans, H].
 __global__ __launch_bounds__(256) void span_states_kernel(ScanArgs a, SpanArgs sp, const int* __restrict__ span_first) {
   const int h = blockIdx.x, r = blockIdx.y, NP = a.N * a.P, i = blockIdx.z * 256 + threadIdx.x;
   if (i >= NP) return;
@@ -395,7 +631,7 @@ __global__ __launch_bounds__(256) void span_states_kernel(ScanArgs a, SpanArgs s
     for (int u = 0; u < 4; ++u) {
       const int c = min(c0 + u, n_spans - 1);
       add[u] = sp.span_state[((size_t)(first + c) * a.H + h) * NP + i];
-      dec[u] = sp.span_decay[(size_t)(first + c) * a.H + h];
+      dec[u] = a.chan_a ? sp.span_decay[((size_t)(first + c) * a.H + h) * a.N + i / a.P] : sp.span_decay[(size_t)(first + c) * a.H + h];
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -505,13 +741,18 @@ static size_t chunk_floats(int N, int P, int C) {
   const size_t Np = (N + 15) & ~15, Pp = (P + 15) & ~15, CP = C + 4;
   return 2 * Np * CP + (size_t)C * Np + 2 * (size_t)C * Pp + (size_t)C * CP + Np * Pp;
 }
+// The same for the kernel with a decay per key channel.
+static size_t channel_chunk_floats(int N, int P, int C) {
+  const size_t Np = (N + 15) & ~15, Pp = (P + 15) & ~15, CP = C + 4;
+  return 3 * Np * CP + 2 * (size_t)C * Pp + (size_t)C * CP + Np * Pp + Np;
+}
 
 // `chunked`: the kernel that takes a chunk of tokens at a time (for steps in which some request
 // brings many tokens); otherwise, or where not even chunks of 16 fit the LDS, token by token.
 // `chunked`: 0 token by token; 1 chunks of tokens, a request a block; 2 chunks, the requests cut
 // into spans of `span` tokens that run side by side (n_spans of them: span_req, span_start; the
 // first span of every request in span_first; span_state: room for n_spans * H * N * P floats,
-// span_decay: for n_spans * H).
+// span_decay: for n_spans * H, with a decay per key channel for n_spans * H * N).
 extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spans, const int* span_req,
                           const int* span_start, const int* span_first, float* span_state, float* span_decay,
                           hipStream_t stream) {
@@ -539,9 +780,11 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
   }
   dim3 grid(a.H, a.n_requests), block(256);
   int C = 0;
-  if (chunked && !a.chan_a)  // (decays per key channel: token by token)
+  // (the chunks with a decay per key channel know neither a scale per token, a skip nor a rotation)
+  const bool by_channel = a.chan_a != nullptr;
+  if (chunked && !(by_channel && (a.k_scale || a.skip || a.rot_dims)))
     for (int c = 64; c >= 16 && !C; c /= 2)
-      if (chunk_floats(a.N, a.P, c) * sizeof(float) <= SCAN_MAX_LDS) C = c;
+      if ((by_channel ? channel_chunk_floats(a.N, a.P, c) : chunk_floats(a.N, a.P, c)) * sizeof(float) <= SCAN_MAX_LDS) C = c;
   if (C) {
     ScanArgs turned = a;  // (the chunked kernel itself turns nothing)
     if (a.rot_dims) {
@@ -556,13 +799,19 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
     if (!chunks_raised) {
       (void)hipFuncSetAttribute((const void*)state_chunks_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
       (void)hipFuncSetAttribute((const void*)state_chunks_kernel<bf16>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
+      (void)hipFuncSetAttribute((const void*)channel_chunks_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
+      (void)hipFuncSetAttribute((const void*)channel_chunks_kernel<bf16>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
       chunks_raised = true;
     }
-    const size_t bytes = chunk_floats(a.N, a.P, C) * sizeof(float);
+    const size_t bytes = (by_channel ? channel_chunk_floats(a.N, a.P, C) : chunk_floats(a.N, a.P, C)) * sizeof(float);
     SpanArgs sp = {WHOLE, 0, nullptr, nullptr, nullptr, nullptr};
 #define CHUNKS(GRID)                                                                                \
   do {                                                                                              \
-    if (a.out_dtype == DT_F32)                                                                      \
+    if (by_channel && a.out_dtype == DT_F32)                                                        \
+      hipLaunchKernelGGL(channel_chunks_kernel<float>, GRID, block, bytes, stream, turned, C, sp);       \
+    else if (by_channel)                                                                            \
+      hipLaunchKernelGGL(channel_chunks_kernel<bf16>, GRID, block, bytes, stream, turned, C, sp);        \
+    else if (a.out_dtype == DT_F32)                                                                 \
       hipLaunchKernelGGL(state_chunks_kernel<float>, GRID, block, bytes, stream, turned, C, sp);         \
     else                                                                                            \
       hipLaunchKernelGGL(state_chunks_kernel<bf16>, GRID, block, bytes, stream, turned, C, sp);          \

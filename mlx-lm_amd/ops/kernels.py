@@ -970,7 +970,7 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
             _dev(t, name, torch.int32)
             _need(t.numel() >= n, f"state_scan: {name} too short")
         ws_state = alloc((n_spans * n_heads * key_dim * value_dim,), torch.float32)
-        ws_decay = alloc((n_spans * n_heads,), torch.float32)
+        ws_decay = alloc((n_spans * n_heads * (key_dim if channel_decay is not None else 1),), torch.float32)
         rc = lib.state_scan(ctypes.byref(a), _c_int(2), _c_int(span), _c_int(n_spans), _ptr(span_req), _ptr(span_start),
                             _ptr(span_first), _ptr(ws_state), _ptr(ws_decay), _stream())
     else:

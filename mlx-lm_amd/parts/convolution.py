@@ -36,6 +36,8 @@ class ShortConvolution(_SequenceArrays, Part):
         import torch
 
         self.weight = torch.cat([tensors[n] for n in self.names]).contiguous()
+        # one tap keeps nothing between steps: the kernel still wants a base address, which it never reads
+        self.no_state = self.weight.new_zeros((1, 1)) if not self.state_floats else None
 
     def state_need(self):
         return StateNeed((self.state_floats,), "float32") if self.state_floats else None
@@ -43,6 +45,8 @@ class ShortConvolution(_SequenceArrays, Part):
     def forward(self, ctx, y, u, state, offset=0):
         """``y`` from ``u`` (float32 rows of ``n_channels`` columns from column 0); ``state``: the
         requests' state rows, this part's floats from ``offset`` on."""
+        if not self.state_floats:
+            state, offset = self.no_state, 0
         starts = ctx.array("sequences.starts")
         single = ctx.array("sequences.longest") == 1
         kernels.causal_conv(y, u, 0, self.weight, None, state, offset, ctx.token_req, starts, ctx.slot_ids,
