@@ -33,7 +33,9 @@ prefill of 2 x 1,024 tokens and decode at batch 1, 8 and 32 from context 512, fo
 ``DESIGN_SIZES`` (``--design-size`` names one, ``--design-only`` one design, for a profile).  The
 Pafutar model runs once without a window (like for like with GPT-2's attention) and once with a
 window of 512 that keeps the first 64 tokens.  Ruzolorn runs at the same layer sizes too
-(``ruzolorn_config``), without a window and with one of 512.  It prints one JSON line of its own.
+(``ruzolorn_config``), without a window and with one of 512, and Zatinex (``zatinex_config``:
+differential attention, gated linear attention and latent attention by turns, a dense gated
+feed-forward).  It prints one JSON line of its own.
 """
 
 import argparse
@@ -71,6 +73,8 @@ def design_config(design, size, window=None):
                     activation_function="gelu_new")
     if design == "ruzolorn":
         return ruzolorn_config(s, window)
+    if design == "zatinex":
+        return zatinex_config(s)
     mixer = {"heads": s["heads"], "kv_heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5}
     if window:
         mixer["mask"] = {"size": window[0], "keep_first": window[1]}
@@ -101,6 +105,41 @@ def ruzolorn_config(s, window=None):
     layers = [dict(retention if i % 2 == 0 else parallel, mlp=mlp) for i in range(s["layers"])]
     return {"architecture": "Ruzolorn", "vocab": DESIGN_VOCAB, "width": D, "max_positions": DESIGN_POSITIONS,
             "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "residual_mult": 0.7, "layers": layers}
+
+
+def zatinex_config(s):
+    """Zatinex at GPT-2's layer sizes, its three mixers by turns.  Differential attention: half as
+    many heads, each with two maps of a head's size over values twice as wide (the projections as
+    large as GPT-2's), four taps, every column turning with interpolated frequencies.  Gated linear
+    attention: as many heads of the same size (Ruzolorn's retention layers at the same sizes are
+    its like), a decay through a middle of 16.  Latent attention: as many heads, a latent of 192
+    columns and half a head of turning ones, queries through a latent of half the width; every
+    second such layer reads the first one's latents.  A gated feed-forward of two thirds of GPT-2's
+    inner size (three matrices where GPT-2 has two)."""
+    H, d, D = s["heads"], s["dim"], s["width"]
+    scaling = {"factor": 4.0, "original": 512, "fast": 32.0, "slow": 1.0}
+    attention = {"type": "attention", "mixer": {"heads": H // 2, "kv_heads": H // 2, "dim": d, "vdim": 2 * d, "conv": 4, "diff": 0.5,
+                                                "scale": d ** -0.5, "rot": {"dims": d, "base": 10000.0, "scaling": scaling}}}
+    gla = {"type": "gla", "mixer": {"heads": H, "dim": d, "vdim": d, "tau": 16.0}}
+    latent = {"heads": H, "dim": d, "rot_dim": d // 2, "vdim": d, "q_rank": D // 2, "kv_rank": 192,
+              "scale": (d + d // 2) ** -0.5, "rot": {"dims": d // 2, "base": 10000.0}}
+    mlp = {"kind": "dense", "ff": s["ff"] * 2 // 3 // 64 * 64}
+    layers, first_latent = [], None
+    for i in range(s["layers"]):
+        if i % 3 == 0:
+            entry = dict(attention)
+        elif i % 3 == 1:
+            entry = dict(gla)
+        else:
+            m = dict(latent)
+            if first_latent is None:
+                first_latent = i
+            elif (i // 3) % 2 == 1:
+                m["kv_from"] = first_latent
+            entry = {"type": "latent_attention", "mixer": m}
+        layers.append(dict(entry, mlp=mlp))
+    return {"architecture": "Zatinex", "vocab": DESIGN_VOCAB, "width": D, "max_positions": DESIGN_POSITIONS,
+            "norm": {"eps": 1e-5}, "layers": layers}
 
 
 def bench_design(config, dtype, batches, steps, warmup):
@@ -150,7 +189,7 @@ def compare_designs(a):
     for size in sizes:
         entry = {"layer_sizes": DESIGN_SIZES[size]}
         runs = {"gpt2": ("gpt2", None), "pafutar": ("pafutar", None), "pafutar_window_512_keep_64": ("pafutar", (512, 64)),
-                "ruzolorn": ("ruzolorn", None), "ruzolorn_window_512": ("ruzolorn", (512, 0))}
+                "ruzolorn": ("ruzolorn", None), "ruzolorn_window_512": ("ruzolorn", (512, 0)), "zatinex": ("zatinex", None)}
         for name, (design, window) in runs.items():
             if a.design_only and name != a.design_only:
                 continue
@@ -259,7 +298,7 @@ def main():
     ap.add_argument("--designs", action="store_true",
                     help="a mode of its own: Pafutar beside GPT-2 at equal layer sizes (prefill and decode)")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default=None, help="with --designs: one size only")
-    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64, ruzolorn, ruzolorn_window_512")
+    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64, ruzolorn, ruzolorn_window_512, zatinex")
     a = ap.parse_args()
     if a.designs:
         if a.gpus != 1:

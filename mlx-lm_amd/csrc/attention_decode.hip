@@ -1,7 +1,7 @@
 // Decode attention: one query row per block, keys streamed from the pages
 // straight into registers (no LDS staging).  bfloat16 caches with head sizes
-// 32, 64 and 128, float caches with 16, 32 and 64 (a lane holds 16 bytes of a
-// key, and 4 to 16 lanes a key).  Same contract as attn_row in attention.hip
+// 32, 64, 128 and 256, float caches with 16, 32, 64 and 128 (a lane holds 16 bytes of a
+// key, and 4 to 32 lanes a key).  Same contract as attn_row in attention.hip
 // (same arguments, same partial buffers, same merge); this is the kernel that
 // serving uses, attn_row stays as the general one (any head size).
 //
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   auto over_groups = [](float v) {
     if (CPK <= 4) v += dpp_move<0x124>(v);  // row_ror:4
     if (CPK <= 8) v += dpp_move<0x128>(v);  // row_ror:8
-    v += __shfl_xor(v, 16, WAVE);
+    if (CPK <= 16) v += __shfl_xor(v, 16, WAVE);
     return v + __shfl_xor(v, 32, WAVE);
   };
   l = over_groups(l);
@@ -374,8 +374,8 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, h
   }
   const size_t lds = p.table_in_lds ? (size_t)p.max_blocks * sizeof(int) : 0;
   const dim3 grid(n_rows, p.n_heads + extra_y, p.n_splits), block(64 * n_waves);
-  if (key_tile == 64)
-    hipLaunchKernelGGL((attn_decode_kernel<T, CPK, 64>), grid, block, lds, stream, p);
+  if (key_tile == 64 && CPK < 32)  // (32 lanes a key: 64 keys would be 64 loads a lane in flight)
+    hipLaunchKernelGGL((attn_decode_kernel<T, (CPK < 32 ? CPK : 16), 64>), grid, block, lds, stream, p);
   else
     hipLaunchKernelGGL((attn_decode_kernel<T, CPK, 32>), grid, block, lds, stream, p);
   if (p.n_splits > 1 && !p.join_here)
@@ -384,8 +384,8 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, h
 
 // Same arguments as attn_row, with what is read ahead and rows_are_requests between: 1 says that
 // item i of `rows` is row i and belongs to request i (every request of the step brings one token),
-// which saves the kernel two trips to memory.  dtype DT_BF16 with head_dim 32, 64 or 128, DT_F32
-// with 16, 32 or 64, and pages that hold whole loads (page_size a multiple of the keys in 1 KB).
+// which saves the kernel two trips to memory.  dtype DT_BF16 with head_dim 32, 64, 128 or 256, DT_F32
+// with 16, 32, 64 or 128, and pages that hold whole loads (page_size a multiple of the keys in 1 KB).
 // key_tile: 32 or 64 keys a wave at a time (0: 32).  join_in_kernel: 0, a second kernel joins the
 // n_splits parts of a (row, head); 1, the block that finishes a (row, head) last does (up to
 // 65,536 (row, head)s; part_o and part_ml are still where the parts pass through); 2, the same,
@@ -409,12 +409,12 @@ extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ld
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("attn_decode: unknown dtype code %d", dtype);
   const int epl = dtype == DT_F32 ? 4 : 8;  // elements in a lane's 16 bytes
   if (n_waves < 1 || n_waves > MAX_WAVES) FAIL("attn_decode: %d waves a block, must be 1 to %d", n_waves, MAX_WAVES);
-  if (head_dim != 4 * epl && head_dim != 8 * epl && head_dim != 16 * epl)
-    FAIL("attn_decode: head_dim %d is not %d, %d or %d (attn_row takes the others)", head_dim, 4 * epl, 8 * epl,
-         16 * epl);
+  if (head_dim != 4 * epl && head_dim != 8 * epl && head_dim != 16 * epl && head_dim != 32 * epl)
+    FAIL("attn_decode: head_dim %d is not %d, %d, %d or %d (attn_row takes the others)", head_dim, 4 * epl, 8 * epl,
+         16 * epl, 32 * epl);
   const int cpk = head_dim / epl;
   if (head_dim > 64 * n_waves) FAIL("attn_decode: head_dim %d needs at least %d waves", head_dim, (head_dim + 63) / 64);
-  if (cpk == 16 && n_waves > MAX_WAVES / 2) n_waves = MAX_WAVES / 2;  // (that kernel's registers allow eight)
+  if (cpk >= 16 && n_waves > MAX_WAVES / 2) n_waves = MAX_WAVES / 2;  // (those kernels' registers allow eight)
   const int kpl = 64 / cpk;
   if (page_size <= 0 || page_size % kpl != 0)
     FAIL("attn_decode: page_size %d must be a multiple of %d for head_dim %d", page_size, kpl, head_dim);
@@ -453,15 +453,19 @@ extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ld
       launch<uint16_t, 4>(p, n_rows, n_waves, key_tile, stream);
     else if (cpk == 8)
       launch<uint16_t, 8>(p, n_rows, n_waves, key_tile, stream);
-    else
+    else if (cpk == 16)
       launch<uint16_t, 16>(p, n_rows, n_waves, key_tile, stream);
+    else
+      launch<uint16_t, 32>(p, n_rows, n_waves, key_tile, stream);
   } else {
     if (cpk == 4)
       launch<float, 4>(p, n_rows, n_waves, key_tile, stream);
     else if (cpk == 8)
       launch<float, 8>(p, n_rows, n_waves, key_tile, stream);
-    else
+    else if (cpk == 16)
       launch<float, 16>(p, n_rows, n_waves, key_tile, stream);
+    else
+      launch<float, 32>(p, n_rows, n_waves, key_tile, stream);
   }
   CHECK_LAUNCH("attn_decode");
   return 0;

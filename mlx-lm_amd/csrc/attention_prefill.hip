@@ -2,7 +2,7 @@
 // prompts, 128 consecutive queries of one request per block, keys and values
 // read from the pages in tiles of 64.  Same contract as attn_tile in
 // attention.hip (same tile list, with up to 128 rows a tile); this is the
-// kernel that serving uses for head sizes 32, 64 and 128, attn_tile stays as
+// kernel that serving uses for head sizes 32, 64, 128 and 256, attn_tile stays as
 // the general one (any head size, float caches).
 //
 // Replaces scaled_dot_product_attention with the "causal" mask and a cache
@@ -405,7 +405,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 
 // tiles: n_tiles pairs (first flat row, number of rows 1..128); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
-// bfloat16 only, head_dim 32, 64 or 128.
+// bfloat16 only, head_dim 32, 64, 128 or 256.
 // attn_prefill_biased: with the optional terms of PrefillArgs (null or 0 where one is absent).
 extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                                    const void* v_pages, size_t page_stride, const int* block_table,
@@ -418,8 +418,8 @@ extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, c
   if (keep_first < 0) FAIL("attn_prefill: keep_first %d must not be negative", keep_first);
   if (gate && (ldg < n_heads * head_dim || ldg % 4 != 0 || ((uintptr_t)gate & 7)))
     FAIL("attn_prefill: the gate's rows (stride %d) must be 8-byte aligned and as wide as the output's", ldg);
-  if (head_dim != 32 && head_dim != 64 && head_dim != 128)
-    FAIL("attn_prefill: head_dim %d is not 32, 64 or 128 (attn_tile takes the others)", head_dim);
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256)
+    FAIL("attn_prefill: head_dim %d is not 32, 64, 128 or 256 (attn_tile takes the others)", head_dim);
   if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
     FAIL("attn_prefill: %d query heads cannot be grouped over %d key heads", n_heads, n_kv_heads);
   if (page_size <= 0) FAIL("attn_prefill: page_size %d must be positive", page_size);
@@ -462,8 +462,10 @@ extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, c
     LAUNCH_PREFILL(32);
   } else if (head_dim == 64) {
     LAUNCH_PREFILL(64);
-  } else {
+  } else if (head_dim == 128) {
     LAUNCH_PREFILL(128);
+  } else {
+    LAUNCH_PREFILL(256);
   }
 #undef LAUNCH_PREFILL
   CHECK_LAUNCH("attn_prefill");

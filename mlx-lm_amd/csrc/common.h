@@ -73,13 +73,15 @@ __device__ __forceinline__ float dpp_move(float v) {
 __device__ __forceinline__ float lane_value(float v, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
-// sum (max) over each group of 4, 8 or 16 neighbouring lanes, in every lane of the group
+// sum (max) over each group of 4, 8 or 16 neighbouring lanes, in every lane of the group (the sum
+// also over 32)
 template <int GROUP>
 __device__ __forceinline__ float group_sum(float v) {
   v += dpp_move<DPP_QUAD_SWAP1>(v);
   v += dpp_move<DPP_QUAD_SWAP2>(v);
   if (GROUP >= 8) v += dpp_move<DPP_HALF_MIRROR>(v);
   if (GROUP >= 16) v += dpp_move<DPP_ROW_MIRROR>(v);
+  if (GROUP >= 32) v += __shfl_xor(v, 16, 64);
   return v;
 }
 template <int GROUP>

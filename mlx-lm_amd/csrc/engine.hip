@@ -751,13 +751,16 @@ struct Attention : Mixer {
     if (n_tiles == 0 && n_rows == 0 && q.rows > 0)
       FAIL("attention: the step carries no work lists for its %d rows", q.rows);
     const bool bf16 = q.dtype == DT_BF16;
-    if (head_dim > ATTN_ROW_MAX_HEAD_DIM) {
+    // (heads of 256 in bfloat16 have the matrix-core and the streaming kernels; other heads wider
+    // than the row kernel takes go to the general tile kernel, rows and all)
+    const bool wide_fast = bf16 && head_dim == 256 && kv.page_size % 2 == 0;
+    if (head_dim > ATTN_ROW_MAX_HEAD_DIM && !wide_fast) {
       KERNEL(k_attn_tile, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks,
              kv.token_req, kv.positions, all_tiles, n_all_tiles, n_heads, n_kv_heads, head_dim, kv.page_size,
              window, scale, q.dtype, ctx->stream);
       return 0;
     }
-    const bool mfma_sizes = bf16 && (head_dim == 32 || head_dim == 64 || head_dim == 128);
+    const bool mfma_sizes = bf16 && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
     if (n_tiles) {
       if (mfma_sizes)
         KERNEL(k_attn_prefill, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
@@ -769,9 +772,9 @@ struct Attention : Mixer {
                kv.page_size, window, scale, q.dtype, ctx->stream);
     }
     if (n_rows) {
-      // the kernel that streams keys into registers: a key in 4, 8 or 16 lanes of 16 bytes
+      // the kernel that streams keys into registers: a key in 4, 8, 16 or 32 lanes of 16 bytes
       const int key_bytes = head_dim * (bf16 ? 2 : 4);
-      const bool fast = (key_bytes == 64 || key_bytes == 128 || key_bytes == 256) &&
+      const bool fast = (key_bytes == 64 || key_bytes == 128 || key_bytes == 256 || key_bytes == 512) &&
                         kv.page_size % (1024 / key_bytes) == 0;
       int n_splits = 1, n_waves = 4, key_tile = 32;
       if (fast)

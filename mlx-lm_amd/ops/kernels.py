@@ -669,11 +669,11 @@ def rows_split_from():
 
 def attn_prefill_takes(q_dtype, kv):
     """Whether the matrix-core prefill kernel takes this cache geometry."""
-    return q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)
+    return q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128, 256)
 
 
 def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0, terms=None):
-    """``attn_tile`` on the matrix cores: bfloat16, head_dim 32/64/128, tiles of up to 128 queries."""
+    """``attn_tile`` on the matrix cores: bfloat16, head_dim 32/64/128/256, tiles of up to 128 queries."""
     lib = build.load("attention_prefill")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
     _need(q.dtype == torch.bfloat16, "attn_prefill: bfloat16 only")
@@ -698,14 +698,14 @@ def attn_decode_takes(q_dtype, kv):
     if q_dtype not in (torch.bfloat16, torch.float32):
         return False
     key_bytes = kv.head_dim * q_dtype.itemsize
-    return key_bytes in (64, 128, 256) and kv.page_size % (1024 // key_bytes) == 0
+    return key_bytes in (64, 128, 256, 512) and kv.page_size % (1024 // key_bytes) == 0
 
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
                 window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0,
                 rows_are_requests=False, key_tile=32, join_in_kernel=0, terms=None):
-    """``attn_row`` for keys of 64, 128 or 256 bytes (bfloat16 with head_dim 32, 64 or 128, float32
-    with 16, 32 or 64): keys stream into registers.
+    """``attn_row`` for keys of 64 to 512 bytes (bfloat16 with head_dim 32, 64, 128 or 256, float32
+    with 16, 32, 64 or 128): keys stream into registers.
 
     ``ahead``: a ``PackedWeight`` whose first ``ahead_chunks`` chunks the CUs without a row read
     meanwhile, each the chunks that a block on its own die will ask for (``sum_partials_norm``).
@@ -1086,6 +1086,19 @@ def head_gate(x, head_stride, n_heads, gate):
                        _c_int(x.shape[0]), _c_int(DT[x.dtype]), _stream())
     build.check(lib, rc, "head_gate")
     return x
+
+
+FAST_HEAD_DIMS = (16, 32, 64, 128, 256)
+
+
+def attention_head_dim(columns):
+    """The head size under which a mixer with heads of ``columns`` columns keeps its pages: the
+    next size that the matrix-core and the streaming attention kernels take (the columns beyond
+    the head's own are zeros in queries, keys and values)."""
+    for n in FAST_HEAD_DIMS:
+        if columns <= n:
+            return n
+    raise ValueError(f"heads of {columns} columns: the attention kernels take at most {FAST_HEAD_DIMS[-1]}")
 
 
 def attend(ctx, out, q, cache, n_heads, n_kv_heads, head_dim, scale, window=0):

@@ -29,7 +29,7 @@ class DifferentialAttention(Mixer):
 
     On the GPU the two maps are two heads of the framework's paged attention: ``2 n_heads`` query
     heads over ``2 n_kv_heads`` key heads of ``head_dim = max(key_dim, value_dim)`` rounded up to
-    16 columns, ordered ``[key head][map][query head of the group]`` so that the kernels' grouping
+    a size that the fast attention kernels take (``kernels.attention_head_dim``), ordered ``[key head][map][query head of the group]`` so that the kernels' grouping
     of query heads over key heads pairs map with map; a key head's values are written beside both
     of its maps' keys.  One product gives ``[q | k | v]`` as float32 rows; convolution, norm and
     rotation are 32-bit (csrc/head_prepare.hip) and write the compute dtype; the attention kernels
@@ -49,9 +49,9 @@ class DifferentialAttention(Mixer):
         n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} query heads cannot be grouped over {n_kv_heads} key heads")
-        self.head_dim = (max(key_dim, value_dim) + 15) // 16 * 16
-        if key_dim <= 0 or value_dim <= 0 or self.head_dim > 256:
+        if key_dim <= 0 or value_dim <= 0 or max(key_dim, value_dim) > 256:
             raise ValueError(f"keys of {key_dim} and values of {value_dim} columns a head (at most 256)")
+        self.head_dim = kernels.attention_head_dim(max(key_dim, value_dim))
         if width % 8:
             raise ValueError(f"width {width} must be a multiple of 8")
         if rot_dims % 2 or not 0 <= rot_dims <= key_dim:

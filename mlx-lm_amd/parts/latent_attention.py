@@ -26,7 +26,7 @@ class LatentAttention(Mixer):
     ``kv_rank`` rows a head beside the ``rot_dim`` rotated ones) and ``Wuv`` into the output
     projection (``Wo_h Wuv_h``) when the weights are loaded, in float64.  The attention is then the
     framework's paged attention with ``n_heads`` query heads over one key head of ``kv_rank +
-    rot_dim`` columns (rounded up to 16; at most 256), whose output's first ``kv_rank`` columns a head
+    rot_dim`` columns (rounded up to a size that the fast attention kernels take; at most 256), whose output's first ``kv_rank`` columns a head
     are the summed latents.  One product gives ``[Wdq x | Wg x | Wdkv x]`` as float32 rows; norms and
     rotation are 32-bit (csrc/head_prepare.hip).  No counterpart in mlx_lm/models/gpt2.py.
     """
@@ -40,11 +40,11 @@ class LatentAttention(Mixer):
     def __init__(self, width, n_heads, key_dim, rot_dim, value_dim, q_rank, kv_rank, scale, eps, rot_base=10000.0,
                  rot_scaling=None, own_latent=True, prefix=""):
         super().__init__(prefix)
-        self.head_dim = (kv_rank + rot_dim + 15) // 16 * 16
         if min(n_heads, key_dim, value_dim, q_rank, kv_rank) <= 0 or rot_dim < 0 or rot_dim % 2:
             raise ValueError(f"{n_heads} heads of {key_dim} + {rot_dim} key and {value_dim} value columns, ranks {q_rank} and {kv_rank}")
-        if self.head_dim > 256:
+        if kv_rank + rot_dim > 256:
             raise ValueError(f"a latent of {kv_rank} + {rot_dim} columns (at most 256 together)")
+        self.head_dim = kernels.attention_head_dim(kv_rank + rot_dim)
         if width % 8:
             raise ValueError(f"width {width} must be a multiple of 8")
         self.width, self.n_heads, self.key_dim, self.rot_dim, self.value_dim = width, n_heads, key_dim, rot_dim, value_dim

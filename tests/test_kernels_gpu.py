@@ -387,11 +387,14 @@ def test_attn_row(dtype, case, n_splits):
 @pytest.mark.parametrize("case", [c for c in ATTN_CASES if c[2] in (32, 64, 128)] + [
     (8, 2, 32, 16, [700, 15, 16], [1, 1, 3], 0),
     (4, 4, 128, 16, [63, 64, 1000], [1, 2, 1], 100),
+    (6, 2, 256, 16, [63, 64, 1000, 0], [1, 2, 1, 1], 0),  # a key in 32 lanes: two keys a load
+    (3, 1, 256, 2, [200, 31], [1, 1], 50),
 ])
 @pytest.mark.parametrize("n_splits,n_waves", [(1, 4), (3, 4), (8, 4), (1, 16), (1, 8), (2, 16), (1, 2)])
 def test_attn_decode(case, n_splits, n_waves):
     k = _k()
     H, Hkv, hd, ps, ctx, ql, window = case
+    n_waves = max(n_waves, hd // 64)  # (a thread a column of the head on the way out)
     c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 2, window=window)
     assert k.attn_decode_takes(torch.bfloat16, c.kv)
     k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
@@ -413,12 +416,14 @@ def test_attn_decode(case, n_splits, n_waves):
     (8, 2, 16, 16, [700, 15, 16], [1, 1, 3], 0),
     (3, 1, 64, 4, [63, 64, 1000], [1, 2, 1], 100),
     (25, 25, 64, 16, [511, 63, 1022, 64, 300], [1, 1, 1, 1, 1], 0),
+    (4, 2, 128, 16, [63, 64, 700], [1, 2, 1], 0),
 ])
 @pytest.mark.parametrize("n_splits,n_waves", [(1, 4), (3, 4), (8, 2), (1, 16), (2, 8), (1, 1)])
 def test_attn_decode_float32(case, n_splits, n_waves):
-    """The same kernel over float caches: a key of 16, 32 or 64 floats in 4, 8 or 16 lanes."""
+    """The same kernel over float caches: a key of 16, 32, 64 or 128 floats in 4, 8, 16 or 32 lanes."""
     k = _k()
     H, Hkv, hd, ps, ctx, ql, window = case
+    n_waves = max(n_waves, hd // 64)
     c = PagedCase(torch.float32, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 3, window=window)
     assert k.attn_decode_takes(torch.float32, c.kv)
     k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
@@ -434,9 +439,9 @@ def test_attn_decode_float32(case, n_splits, n_waves):
         assert err < _attn_tol(torch.float32), (key_tile, here, err)
 
 
-def test_attn_decode_takes_keys_of_64_to_256_bytes():
+def test_attn_decode_takes_keys_of_64_to_512_bytes():
     k = _k()
-    for dtype, hd, ps, takes in [(torch.float32, 128, 16, False), (torch.float32, 48, 16, False),
+    for dtype, hd, ps, takes in [(torch.float32, 256, 16, False), (torch.float32, 48, 16, False), (torch.bfloat16, 256, 2, True),
                                  (torch.float32, 64, 2, False), (torch.float32, 64, 4, True),
                                  (torch.float32, 16, 16, True), (torch.bfloat16, 16, 16, False),
                                  (torch.bfloat16, 128, 4, True), (torch.bfloat16, 32, 8, False)]:
@@ -484,6 +489,8 @@ PREFILL_CASES = [c for c in ATTN_CASES if c[2] in (32, 64, 128)] + [
     (5, 5, 64, 16, [0, 400], [333, 128], 90),
     (2, 2, 64, 48, [30, 0], [200, 150], 0),  # a page size that is no power of two
     (3, 1, 32, 80, [0, 77], [170, 40], 60),
+    (4, 2, 256, 16, [0, 100, 300], [300, 129, 5], 0),
+    (2, 1, 256, 48, [30, 0], [200, 150], 70),
 ]
 
 

@@ -69,8 +69,8 @@ def test_the_plan_run_by_run():
     assert [(r.layer, r.cache, r.writes_cache, r.state) for r in runs] == [
         (0, 0, True, None), (1, 1, True, 2), (2, 3, True, None), (3, 0, False, None), (4, 4, True, None)]
     needs = model.decoder.cache_needs()
-    assert needs[0] == CacheNeed(1, 48, 0)  # one key head of kv_rank + rot_dim columns
-    assert needs[1] == CacheNeed(6, 32, 0)  # two maps of three key heads, max(16, 24) rounded up to 16s
+    assert needs[0] == CacheNeed(1, 64, 0)  # one key head of kv_rank + rot_dim = 48 columns, in the next size the kernels take
+    assert needs[1] == CacheNeed(6, 32, 0)  # two maps of three key heads, max(16, 24) in the next size
     assert needs[2] == StateNeed(((4 - 1) * (2 * 6 * 16 + 2 * 3 * 16 + 3 * 24),), "float32")
     assert needs[3] == StateNeed((2 * 24 * 16,), "float32") and needs[4] == StateNeed((4 * 8 * 8,), "float32")
     names = model.decoder.expected_tensors()
