@@ -14,6 +14,7 @@
 //                   sin times `rot_mult`; then the head goes to `copies` places: copy c of head h
 //                   to column dst_head[c * n_heads + h] * dst_stride of the output row (h itself
 //                   without a table), zeros from `dim` up to `dst_fill` columns.
+//                   head_prepare_many: up to four such preparations in one launch.
 //   diff_combine    o = a1 - lambda a2 per head, where a1 and a2 are two heads of an attention's
 //                   output (tables say which), divided by its root mean square and multiplied by
 //                   `mult`.
@@ -64,9 +65,7 @@ struct PrepareArgs {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void head_prepare_kernel(PrepareArgs a) {
-  const int lane = threadIdx.x & 63;
-  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+__device__ __forceinline__ void prepare_head(const PrepareArgs& a, long item, int lane) {
   if (item >= (long)a.n_rows * a.n_heads) return;  // whole waves leave; no barrier follows
   const int row = (int)(item / a.n_heads), h = (int)(item % a.n_heads);
   const float* s = a.src + (size_t)row * a.lds + a.src_col + (size_t)h * a.src_stride;
@@ -103,6 +102,27 @@ __global__ __launch_bounds__(256) void head_prepare_kernel(PrepareArgs a) {
       ((T*)a.dst)[(size_t)row * a.ldd + (size_t)dh * a.dst_stride + k] = from_f32<T>(v);
     }
   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void head_prepare_kernel(PrepareArgs a) {
+  prepare_head<T>(a, (long)blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & 63);
+}
+
+// Several preparations in one launch (a mixer's queries, keys and values): the blocks of each
+// follow those of the one before.
+#define PREPARE_MOST 4
+struct PrepareMany {
+  PrepareArgs seg[PREPARE_MOST];
+  unsigned first_block[PREPARE_MOST + 1];
+  int n;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void head_prepare_many_kernel(PrepareMany m) {
+  int s = 0;
+  while (s + 1 < m.n && blockIdx.x >= m.first_block[s + 1]) ++s;
+  prepare_head<T>(m.seg[s], (long)(blockIdx.x - m.first_block[s]) * 4 + (threadIdx.x >> 6), threadIdx.x & 63);
 }
 
 // A wave a (row, head).
@@ -157,9 +177,7 @@ extern "C" int causal_conv(const float* u, int ldu, int col, const float* w, con
   return 0;
 }
 
-extern "C" int head_prepare(const PrepareArgs* args, int dst_dtype, hipStream_t stream) {
-  const PrepareArgs& a = *args;
-  if (a.n_rows <= 0 || a.n_heads <= 0) return 0;
+static int prepare_args_fit(const PrepareArgs& a) {
   if (!a.src || !a.dst) FAIL("head_prepare: null pointer");
   if (a.dim <= 0 || a.src_col < 0 || a.src_col + (long)(a.n_heads - 1) * a.src_stride + a.dim > a.lds)
     FAIL("head_prepare: %d heads of %d columns, %d apart from column %d, in rows of %d", a.n_heads, a.dim, a.src_stride,
@@ -171,6 +189,13 @@ extern "C" int head_prepare(const PrepareArgs* args, int dst_dtype, hipStream_t 
     FAIL("head_prepare: %d copies, %d columns filled of %d, a head of %d", a.copies, a.dst_fill, a.dst_stride, a.dim);
   if (!a.dst_head && (a.copies != 1 || (long)(a.n_heads - 1) * a.dst_stride + a.dst_fill > a.ldd))
     FAIL("head_prepare: the heads do not fit rows of %d", a.ldd);
+  return 0;
+}
+
+extern "C" int head_prepare(const PrepareArgs* args, int dst_dtype, hipStream_t stream) {
+  const PrepareArgs& a = *args;
+  if (a.n_rows <= 0 || a.n_heads <= 0) return 0;
+  if (prepare_args_fit(a)) return 1;
   if (dst_dtype != DT_F32 && dst_dtype != DT_BF16) FAIL("head_prepare: unknown dtype code %d", dst_dtype);
   const long items = (long)a.n_rows * a.n_heads;
   dim3 grid((unsigned)((items + 3) / 4)), block(256);
@@ -179,6 +204,31 @@ extern "C" int head_prepare(const PrepareArgs* args, int dst_dtype, hipStream_t 
   else
     hipLaunchKernelGGL(head_prepare_kernel<bf16>, grid, block, 0, stream, a);
   CHECK_LAUNCH("head_prepare");
+  return 0;
+}
+
+// `n` preparations (1 to 4) whose outputs are all of `dst_dtype`, in one launch.
+extern "C" int head_prepare_many(const PrepareArgs* args, int n, int dst_dtype, hipStream_t stream) {
+  if (n < 1 || n > PREPARE_MOST || !args) FAIL("head_prepare_many: %d preparations (1 to %d)", n, PREPARE_MOST);
+  if (dst_dtype != DT_F32 && dst_dtype != DT_BF16) FAIL("head_prepare: unknown dtype code %d", dst_dtype);
+  PrepareMany m;
+  m.n = 0;
+  unsigned blocks = 0;
+  for (int i = 0; i < n; ++i) {
+    const PrepareArgs& a = args[i];
+    if (a.n_rows <= 0 || a.n_heads <= 0) continue;
+    if (prepare_args_fit(a)) return 1;
+    m.seg[m.n] = a, m.first_block[m.n] = blocks;
+    blocks += (unsigned)(((long)a.n_rows * a.n_heads + 3) / 4);
+    ++m.n;
+  }
+  if (m.n == 0) return 0;
+  for (int i = m.n; i <= PREPARE_MOST; ++i) m.first_block[i] = blocks;
+  if (dst_dtype == DT_F32)
+    hipLaunchKernelGGL(head_prepare_many_kernel<float>, dim3(blocks), dim3(256), 0, stream, m);
+  else
+    hipLaunchKernelGGL(head_prepare_many_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, m);
+  CHECK_LAUNCH("head_prepare_many");
   return 0;
 }
 

@@ -1019,9 +1019,7 @@ class PrepareArgs(ctypes.Structure):
                 ("dst_fill", _c_int), ("copies", _c_int), ("dst_head", _vp)]
 
 
-def head_prepare(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=None, dst_fill=None, norm_dim=0,
-                 norm_weight=None, eps=0.0, rot_off=0, rot_dims=0, inv_freq=None, rot_mult=1.0, interleaved=True,
-                 positions=None, dst_head=None, copies=1):
+def head_prepare(dst, src, src_col, n_heads, dim, **options):
     """Heads of a float32 projection row on their way to an attention: head ``h`` is ``dim`` columns
     of ``src`` from ``src_col + h * src_stride``; RMS norm over its first ``norm_dim`` columns
     (times ``norm_weight``, shared by the heads); rotation of ``rot_dims`` columns from ``rot_off``
@@ -1030,6 +1028,25 @@ def head_prepare(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=No
     column ``dst_head[c, h] * dst_stride`` for each of ``copies`` copies (``h * dst_stride`` without
     a table), with zeros from ``dim`` up to ``dst_fill`` columns."""
     lib = build.load("head_prepare")
+    a = _prepare_args(dst, src, src_col, n_heads, dim, **options)
+    rc = lib.head_prepare(ctypes.byref(a), _c_int(DT[dst.dtype]), _stream())
+    build.check(lib, rc, "head_prepare")
+    return dst
+
+
+def head_prepare_many(*calls):
+    """Several ``head_prepare`` calls in one launch: each of ``calls`` is ``(dst, src, src_col,
+    n_heads, dim, options)``; at most four, their ``dst`` of one dtype."""
+    lib = build.load("head_prepare")
+    _need(1 <= len(calls) <= 4 and len({c[0].dtype for c in calls}) == 1, "head_prepare_many: one to four calls, outputs of one dtype")
+    args = (PrepareArgs * len(calls))(*[_prepare_args(*c[:5], **c[5]) for c in calls])
+    rc = lib.head_prepare_many(args, _c_int(len(calls)), _c_int(DT[calls[0][0].dtype]), _stream())
+    build.check(lib, rc, "head_prepare_many")
+
+
+def _prepare_args(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=None, dst_fill=None, norm_dim=0,
+                  norm_weight=None, eps=0.0, rot_off=0, rot_dims=0, inv_freq=None, rot_mult=1.0, interleaved=True,
+                  positions=None, dst_head=None, copies=1):
     a = PrepareArgs()
     src_stride = dim if src_stride is None else src_stride
     dst_stride = dim if dst_stride is None else dst_stride
@@ -1056,9 +1073,7 @@ def head_prepare(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=No
         _need(dst_head.numel() == copies * n_heads, "head_prepare: dst_head is [copies, heads]")
         a.dst_head = dst_head.data_ptr()
     _need(dst.shape[1] >= (n_heads * copies - 1) * dst_stride + a.dst_fill, "head_prepare: dst rows are too short for the heads")
-    rc = lib.head_prepare(ctypes.byref(a), _c_int(DT[dst.dtype]), _stream())
-    build.check(lib, rc, "head_prepare")
-    return dst
+    return a
 
 
 def diff_combine(out, att, head_stride, first, second, lam, mult, eps, vdim):

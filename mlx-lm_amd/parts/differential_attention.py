@@ -121,15 +121,17 @@ class DifferentialAttention(Mixer):
             u = y
         rot = dict(rot_dims=self.rot_dims, inv_freq=self.inv_freq, rot_mult=self.rot_mult, positions=ctx.positions)
         q = ctx.scratch((T, H2 * hd), ctx.dtype)
-        kernels.head_prepare(q, u, 0, H2, d, dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.q_norm, eps=self.eps,
-                             dst_head=self.q_place, **rot)
+        calls = [(q, u, 0, H2, d, dict(dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.q_norm, eps=self.eps,
+                                       dst_head=self.q_place, **rot))]
         if writes_cache:
             k = ctx.scratch((T, G2 * hd), ctx.dtype)
             v = ctx.scratch((T, G2 * hd), ctx.dtype)
-            kernels.head_prepare(k, u, self.q_cols, G2, d, dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.k_norm,
-                                 eps=self.eps, **rot)
-            kernels.head_prepare(v, u, self.q_cols + self.k_cols, self.n_kv_heads, self.value_dim, dst_stride=hd, dst_fill=hd,
-                                 dst_head=self.v_place, copies=2)
+            calls.append((k, u, self.q_cols, G2, d, dict(dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.k_norm,
+                                                         eps=self.eps, **rot)))
+            calls.append((v, u, self.q_cols + self.k_cols, self.n_kv_heads, self.value_dim,
+                          dict(dst_stride=hd, dst_fill=hd, dst_head=self.v_place, copies=2)))
+        kernels.head_prepare_many(*calls)  # (queries, keys and values in one launch)
+        if writes_cache:
             kernels.kv_write(k, v, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
         att = ctx.scratch((T, H2 * hd), ctx.dtype)
         kernels.attend(ctx, att, q, cache, H2, G2, hd, self.scale)

@@ -103,13 +103,15 @@ class LatentAttention(Mixer):
         kernels.linear(qf, cq, self.q_w, splits=kernels.splits_alone(T))
         rot = dict(rot_off=r, rot_dims=dr, inv_freq=self.inv_freq, rot_mult=self.rot_mult, positions=ctx.positions)
         q = ctx.scratch((T, H * hd), ctx.dtype)
-        kernels.head_prepare(q, qf, 0, H, r + dr, dst_stride=hd, dst_fill=hd, **rot)
+        calls = [(q, qf, 0, H, r + dr, dict(dst_stride=hd, dst_fill=hd, **rot))]
         if writes_cache:
             if not self.own_latent:
                 raise RuntimeError("a latent-attention layer without a down-projection reads another layer's cache slot")
             c = ctx.scratch((T, hd), ctx.dtype)
-            kernels.head_prepare(c, u, Q + H, 1, r + dr, dst_stride=hd, dst_fill=hd, norm_dim=r, norm_weight=self.c_norm,
-                                 eps=self.eps, **rot)
+            calls.append((c, u, Q + H, 1, r + dr, dict(dst_stride=hd, dst_fill=hd, norm_dim=r, norm_weight=self.c_norm,
+                                                       eps=self.eps, **rot)))
+        kernels.head_prepare_many(*calls)  # (queries and the latent in one launch)
+        if writes_cache:
             kernels.kv_write(c, c, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
         att = ctx.scratch((T, H * hd), ctx.dtype)
         kernels.attend(ctx, att, q, cache, H, 1, hd, self.scale)
