@@ -76,6 +76,11 @@ __device__ __forceinline__ float gate_at(const DecodeArgs& p, int row, int col) 
 
 #define MAX_WAVES 16
 
+union Frag8g {
+  uint4 u;
+  bf16x8_t v;
+};
+
 // ldo == 0: out is in the packed order, tiles of 16 rows x 64 columns
 __device__ __forceinline__ size_t out_at(const DecodeArgs& p, int row, int col) {
   return p.ldo != 0 ? (size_t)row * p.ldo + col : packed_at(row, col, (p.n_heads * p.out_head_dim + 63) / 64);
@@ -342,6 +347,147 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   }
 }
 
+// attn_decode_group: bfloat16, the query heads that share a key head taken together.  Where many
+// query heads read one key head (a latent that all heads share, large groups), a block a (row,
+// head) walks the same keys once a head and pays a key's instructions each time.  Here a block
+// takes a (row, key head, sixteen of its query heads, part of the keys), a wave sixteen keys at a
+// time, on the matrix cores:
+//   S^T = K Q^T   v_mfma_f32_16x16x32_bf16: keys are the rows (lane l brings 16 bytes of key l % 16
+//                 straight from its page), the heads the columns (the queries stay in registers);
+//                 a lane then holds four keys' scores of head l % 16.
+//   O^T += V^T P^T  v_mfma_f32_16x16x16_bf16: those four weights are the lane's fragment of P^T as
+//                 they are; the lane brings column 16 d + l % 16 of its four keys' values.
+// Online softmax per head in 32-bit; the waves' results are joined through LDS in the waves'
+// order, the parts of a split row by attn_decode_merge_kernel.
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_group_kernel(DecodeArgs p, int group, int head_tiles) {
+  constexpr int QC = HD / 32;      // steps of K Q^T
+  constexpr int DT = HD / 16;      // 16-row tiles of O^T
+  constexpr int OS = HD + 1;       // a head's row in Os (the odd stride keeps sixteen heads on sixteen banks)
+  __shared__ float Ms[4][16], Ls[4][16];
+  extern __shared__ int group_lds[];
+  float* Os = (float*)group_lds;                 // [4 waves][16 heads][OS]
+  int* pages = group_lds + 4 * 16 * OS;          // [max_blocks] with table_in_lds
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c16 = lane & 15;
+  const int item = blockIdx.x, split = blockIdx.z;
+  const int kv_head = blockIdx.y / head_tiles, ht = blockIdx.y % head_tiles;
+  const int row = p.rows_are_requests ? item : p.rows[item];
+  const int req = p.rows_are_requests ? item : p.token_req[row];
+  const int* table = p.block_table + (size_t)req * p.max_blocks;
+  if (p.table_in_lds)
+    for (int i = tid; i < p.max_blocks; i += 256) pages[i] = table[i];
+  const int pos = p.positions[row];
+  const uint16_t* k_pages = (const uint16_t*)p.k_pages;
+  const uint16_t* v_pages = (const uint16_t*)p.v_pages;
+  const int in_group = ht * 16 + c16;  // this lane's head within the group
+  const int head = kv_head * group + min(in_group, group - 1);
+  Frag8g qf[QC];
+  {
+    const uint16_t* qrow = (const uint16_t*)p.q + (size_t)row * p.ldq + (size_t)head * HD + 8 * g;
+#pragma unroll
+    for (int c = 0; c < QC; ++c) {
+      qf[c].u = *(const uint4*)(qrow + 32 * c);
+      if (in_group >= group) qf[c].u = make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+  const int k_hi = pos + 1;
+  const int k_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int kt0 = (k_lo / 16) * 16;
+  const int n_tiles = (k_hi - kt0 + 15) / 16;
+  const int per_split = (n_tiles + p.n_splits - 1) / p.n_splits;
+  const int t_begin = split * per_split, t_end = min(n_tiles, t_begin + per_split);
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const size_t head_off = (size_t)kv_head * p.page_size * HD;
+  if (p.table_in_lds) __syncthreads();  // (uniform over the block)
+  auto page_of_key = [&](int key) { return p.table_in_lds ? pages[key / p.page_size] : table[key / p.page_size]; };
+
+  for (int t = t_begin + wave; t < t_end; t += 4) {
+    const int kt = kt0 + t * 16;
+    Frag8g kf[QC];
+    {
+      const int key = min(max(kt + c16, k_lo), k_hi - 1);  // (keys outside the run: pulled inside, masked below)
+      const uint16_t* kp = k_pages + (size_t)page_of_key(key) * p.page_stride + head_off + (size_t)(key % p.page_size) * HD + 8 * g;
+#pragma unroll
+      for (int c = 0; c < QC; ++c) kf[c].u = *(const uint4*)(kp + 32 * c);
+    }
+    const uint16_t* vp[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int key = min(max(kt + 4 * g + x, k_lo), k_hi - 1);
+      vp[x] = v_pages + (size_t)page_of_key(key) * p.page_stride + head_off + (size_t)(key % p.page_size) * HD + c16;
+    }
+    s16x4_t va[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int x = 0; x < 4; ++x) va[d][x] = (short)vp[x][16 * d];
+    f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < QC; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c].v, qf[c].v, s, 0, 0, 0);
+    float sx[4], tmax = -INFINITY;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int key = kt + 4 * g + x;
+      sx[x] = (key >= k_lo && key < k_hi) ? s[x] * p.scale : -INFINITY;
+      tmax = fmaxf(tmax, sx[x]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(m, tmax);  // finite: every tile holds at least one live key
+    const float alpha = __expf(m - m_new);
+    s16x4_t pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const float px = __expf(sx[x] - m_new);  // exp(-inf) = 0 for masked keys
+      psum += px;
+      pb[x] = (short)f32_to_bf16_bits(px);
+    }
+    l = l * alpha + psum;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) o[d][x] *= alpha;
+      o[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[d], pb, o[d], 0, 0, 0);
+    }
+    m = m_new;
+  }
+  // the four lane groups of a head hold sums over different keys
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (g == 0) Ms[wave][c16] = m, Ls[wave][c16] = l;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) Os[((size_t)wave * 16 + c16) * OS + 16 * d + 4 * g + x] = o[d][x];
+  __syncthreads();
+  for (int e = tid; e < 16 * HD; e += 256) {
+    const int hh = e / HD, col = e - hh * HD;
+    if (ht * 16 + hh >= group) continue;
+    float M = -INFINITY;
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, Ms[w][hh]);
+    float L = 0.f, acc = 0.f;
+    for (int w = 0; w < 4; ++w) {
+      const float f = (Ms[w][hh] == -INFINITY) ? 0.f : __expf(Ms[w][hh] - M);
+      L += Ls[w][hh] * f;
+      acc += Os[((size_t)w * 16 + hh) * OS + col] * f;
+    }
+    const int hq = kv_head * group + ht * 16 + hh;
+    if (p.n_splits == 1) {
+      put((uint16_t*)p.out + out_at(p, row, hq * HD + col), acc / L);
+    } else {
+      const size_t base = ((size_t)item * p.n_heads + hq) * p.n_splits + split;
+      p.part_o[base * HD + col] = acc;
+      if (col == 0) p.part_ml[base * 2] = M, p.part_ml[base * 2 + 1] = L;
+    }
+  }
+}
+
 // grid (rows, heads), HD threads: join the splits
 template <typename T, int CPK>
 __global__ void attn_decode_merge_kernel(DecodeArgs p) {
@@ -484,4 +630,60 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
                                  n_splits, part_o, part_ml, n_waves, ahead, ahead_chunk_bytes, ahead_chunks,
                                  rows_are_requests, dtype, key_tile, join_in_kernel, nullptr, nullptr, nullptr, 0, 0,
                                  stream);
+}
+
+// attn_decode_group: the rows of attn_decode_rows for bfloat16 caches with head_dim 64, 128 or 256,
+// all query heads of a key head in one block (see attn_decode_group_kernel).  n_splits parts of a
+// row's keys (part_o: n_rows * n_heads * n_splits * head_dim floats, part_ml: two a part; joined
+// by a second kernel).  ldo == 0: out in the packed order.
+extern "C" int attn_decode_group(void* out, const void* q, int ldq, int ldo, const void* k_pages, const void* v_pages,
+                                 size_t page_stride, const int* block_table, int max_blocks, const int* token_req,
+                                 const int* positions, const int* rows, int n_rows, int n_heads, int n_kv_heads,
+                                 int head_dim, int page_size, int window, float scale, int n_splits, float* part_o,
+                                 float* part_ml, int rows_are_requests, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) FAIL("attn_decode_group: head_dim %d is not 64, 128 or 256", head_dim);
+  if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
+    FAIL("attn_decode_group: %d query heads cannot be grouped over %d key heads", n_heads, n_kv_heads);
+  if (!out || !q || !k_pages || !v_pages || !block_table || !token_req || !positions || !rows)
+    FAIL("attn_decode_group: null pointer");
+  if (page_size <= 0 || window < 0) FAIL("attn_decode_group: page_size %d, window %d", page_size, window);
+  if (ldq % 8 != 0 || ((uintptr_t)q & 15)) FAIL("attn_decode_group: queries must be 16-byte aligned rows");
+  if (page_stride % 8 != 0 || (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
+    FAIL("attn_decode_group: pages must be 16-byte aligned");
+  if (n_splits < 1 || n_splits > 65535) FAIL("attn_decode_group: %d parts", n_splits);
+  if (n_splits > 1 && (!part_o || !part_ml)) FAIL("attn_decode_group: parts need part_o and part_ml");
+  DecodeArgs p = {};
+  p.out = out, p.q = q, p.k_pages = k_pages, p.v_pages = v_pages;
+  p.block_table = block_table, p.token_req = token_req, p.positions = positions, p.rows = rows;
+  p.part_o = part_o, p.part_ml = part_ml, p.page_stride = page_stride;
+  p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
+  p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size, p.window = window, p.n_splits = n_splits;
+  p.scale = scale, p.out_head_dim = head_dim, p.rows_are_requests = rows_are_requests ? 1 : 0;
+  p.table_in_lds = max_blocks > 0 && max_blocks <= 8192;
+  const int group = n_heads / n_kv_heads, head_tiles = (group + 15) / 16;
+  if ((long)n_kv_heads * head_tiles > 65535) FAIL("attn_decode_group: %d key heads in a launch", n_kv_heads);
+  const size_t lds = (size_t)4 * 16 * (head_dim + 1) * sizeof(float) + (p.table_in_lds ? (size_t)max_blocks * sizeof(int) : 0);
+  const dim3 grid(n_rows, n_kv_heads * head_tiles, n_splits), block(256);
+#define LAUNCH_GROUP(HD)                                                                                             \
+  do {                                                                                                               \
+    static bool raised = false;                                                                                      \
+    if (!raised) {                                                                                                   \
+      (void)hipFuncSetAttribute((const void*)attn_decode_group_kernel<HD>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                120 * 1024);                                                                         \
+      raised = true;                                                                                                 \
+    }                                                                                                                \
+    hipLaunchKernelGGL((attn_decode_group_kernel<HD>), grid, block, lds, stream, p, group, head_tiles);              \
+    if (n_splits > 1)                                                                                                \
+      hipLaunchKernelGGL((attn_decode_merge_kernel<uint16_t, HD / 8>), dim3(n_rows, n_heads), dim3(HD), 0, stream, p); \
+  } while (0)
+  if (head_dim == 64)
+    LAUNCH_GROUP(64);
+  else if (head_dim == 128)
+    LAUNCH_GROUP(128);
+  else
+    LAUNCH_GROUP(256);
+#undef LAUNCH_GROUP
+  CHECK_LAUNCH("attn_decode_group");
+  return 0;
 }

@@ -111,6 +111,9 @@ typedef int (*fn_attn_row)(void*, const void*, int, int, const void*, const void
 typedef int (*fn_attn_decode)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
                               const int*, const int*, const int*, int, int, int, int, int, int, float, int,
                               float*, float*, int, const void*, size_t, int, int, int, int, int, hipStream_t);
+typedef int (*fn_attn_decode_group)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
+                                    const int*, const int*, const int*, int, int, int, int, int, int, float, int,
+                                    float*, float*, int, hipStream_t);
 typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const void*, size_t, const int*,
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
@@ -135,6 +138,7 @@ static Entry<fn_kv_write> k_kv_write("attention", "kv_write");
 static Entry<fn_attn_tile> k_attn_tile("attention", "attn_tile");
 static Entry<fn_attn_row> k_attn_row("attention", "attn_row");
 static Entry<fn_attn_decode> k_attn_decode("attention_decode", "attn_decode_rows");
+static Entry<fn_attn_decode_group> k_attn_decode_group("attention_decode", "attn_decode_group");
 static Entry<fn_attn_prefill> k_attn_prefill("attention_prefill", "attn_prefill");
 
 // Launch through an entry: a missing library or a refused call becomes this library's error.
@@ -777,6 +781,30 @@ struct Attention : Mixer {
       const bool fast = (key_bytes == 64 || key_bytes == 128 || key_bytes == 256 || key_bytes == 512) &&
                         kv.page_size % (1024 / key_bytes) == 0;
       int n_splits = 1, n_waves = 4, key_tile = 32;
+      // eight or more query heads a key head (a latent that all heads share): the kernel that takes
+      // them together on the matrix cores, so a key is read and multiplied once for all of them.
+      // A block is four waves of sixteen keys at a time; a part for every 128 keys of the longest
+      // row, as many as give every CU two blocks.
+      const int group = n_heads / n_kv_heads;
+      if (bf16 && group >= 8 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
+        const long c = window <= 0 ? max_row_context : (max_row_context < window + 15 ? max_row_context : window + 15);
+        const long blocks = (long)n_rows * n_kv_heads * ((group + 15) / 16);
+        long ns = c / 128, most = 2L * ctx->n_compute_units / (blocks < 1 ? 1 : blocks);
+        if (ns > most) ns = most;
+        if (ns > 64) ns = 64;
+        if (ns < 1) ns = 1;
+        if (ctx->stats && ns > ctx->stats->key_splits_most) ctx->stats->key_splits_most = (int)ns;
+        EngMat group_o = {}, group_ml = {};
+        if (ns > 1) {
+          const long n = (long)n_rows * n_heads * ns;
+          TRY(take(ctx, 1, (int)(n * head_dim), DT_F32, &group_o));
+          TRY(take(ctx, 1, (int)(n * 2), DT_F32, &group_ml));
+        }
+        KERNEL(k_attn_decode_group, ctx, out.p, q.p, q.ld, out_packed ? 0 : out.ld, kv.k, kv.v, kv.page_stride,
+               kv.block_table, kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
+               kv.page_size, window, scale, (int)ns, (float*)group_o.p, (float*)group_ml.p, rows_are_requests, ctx->stream);
+        return 0;
+      }
       if (fast)
         row_work(ctx, n_rows, max_row_context, &n_splits, &n_waves, &key_tile);
       else

@@ -747,6 +747,34 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
     return out
 
 
+def attn_decode_group(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale, window=0, n_splits=1,
+                      part_o=None, part_ml=None, rows_are_requests=False):
+    """``attn_row`` for bfloat16 caches with head_dim 64, 128 or 256 where many query heads share a key
+    head: a block takes sixteen query heads of a key head at once, on the matrix cores, so a key is
+    read once for all of them.  ``n_splits`` parts of a row's keys, joined by a second kernel."""
+    lib = build.load("attention_decode")
+    ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
+    _need(q.dtype == torch.bfloat16 and out.dtype == q.dtype, "attn_decode_group: bfloat16 only")
+    _need(q.shape[1] == n_heads * kv.head_dim and out.shape[1] == q.shape[1], "attn_decode_group: rows of n_heads*head_dim")
+    _attn_common(q, kv, block_table, token_req, positions)
+    _dev(rows, "rows", torch.int32)
+    _need(rows.numel() >= n_rows, "attn_decode_group: row list too short")
+    if n_splits > 1:
+        _dev(part_o, "part_o", torch.float32)
+        _dev(part_ml, "part_ml", torch.float32)
+        _need(part_o.numel() >= n_rows * n_heads * n_splits * kv.head_dim, "attn_decode_group: part_o too small")
+        _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_decode_group: part_ml too small")
+    if rows_are_requests:
+        _need(n_rows <= block_table.shape[0], "attn_decode_group: more rows than requests")
+    rc = lib.attn_decode_group(
+        _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v), _c_size_t(kv.page_stride), _ptr(block_table),
+        _c_int(block_table.shape[1]), _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
+        _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window), _c_float(scale), _c_int(n_splits),
+        _ptr(part_o), _ptr(part_ml), _c_int(1 if rows_are_requests else 0), _stream())
+    build.check(lib, rc, "attn_decode_group")
+    return out
+
+
 # ---------------------------------------------------------------------------
 
 

@@ -439,6 +439,31 @@ def test_attn_decode_float32(case, n_splits, n_waves):
         assert err < _attn_tol(torch.float32), (key_tile, here, err)
 
 
+@pytest.mark.parametrize("case", [
+    (16, 1, 256, 16, [700, 15, 16, 0], [1, 1, 3, 1], 0),   # sixteen heads over one latent
+    (24, 2, 64, 16, [63, 64, 1000], [1, 2, 1], 100),        # twelve heads a key head: four empty columns of the tile
+    (40, 2, 128, 8, [300, 5], [1, 1], 0),                   # twenty heads a key head: two tiles of heads
+    (8, 1, 128, 48, [200, 31], [2, 1], 50),                 # a page size that is no power of two
+])
+@pytest.mark.parametrize("n_splits", [1, 3, 8])
+def test_attn_decode_group(case, n_splits):
+    """All query heads of a key head in one block on the matrix cores, against the same reference
+    as the other decode kernels; rows told to be requests or looked up."""
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 7, window=window)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
+    part_o = torch.full((c.T * H * n_splits * hd,), float("nan"), dtype=torch.float32, device=DEV)
+    part_ml = torch.full((c.T * H * n_splits * 2,), float("nan"), dtype=torch.float32, device=DEV)
+    want = c.reference()
+    out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
+    k.attn_decode_group(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H, c.scale, window,
+                        n_splits, part_o, part_ml)
+    err = (out.double().cpu() - want).abs().max().item()
+    assert err < _attn_tol(torch.bfloat16), err
+
+
 def test_attn_decode_takes_keys_of_64_to_512_bytes():
     k = _k()
     for dtype, hd, ps, takes in [(torch.float32, 256, 16, False), (torch.float32, 48, 16, False), (torch.bfloat16, 256, 2, True),
