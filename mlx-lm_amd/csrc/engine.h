@@ -122,6 +122,9 @@ typedef struct {
   EngMat result;
   const int* index;
   size_t nbytes;  // ENG_CB_GROW: what the scratch buffer has to hold
+  // a mixer's or feed-forward's input as a norm that is not computed yet (for a part made with
+  // ENG_ACCEPTS_LAZY; x.p is null then, x says the shape)
+  EngValue x_lazy;
 } EngCall;
 
 enum {

@@ -120,6 +120,7 @@ typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const 
 
 static Entry<fn_embed> k_embed("embed", "embed_scale_add");
 static Entry<fn_layernorm> k_layernorm("norm", "layernorm");
+static Entry<int (*)(void*, const float*, int, const int*, const float*, float, int, int, int, hipStream_t)> k_rmsnorm("rmsnorm", "rmsnorm");
 static Entry<fn_gemm_f32> k_gemm_f32("gemm_f32", "gemm_f32");
 static Entry<fn_int4> k_gemm_f32_splits("gemm_f32", "gemm_f32_splits");
 static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16_scatter");
@@ -296,6 +297,10 @@ static int materialize(EngCtx* ctx, const EngValue& v, EngMat* out) {
   }
   if (v.ldx != v.m.cols) FAIL("a lazy norm's rows must be contiguous");
   TRY(take(ctx, v.m.rows, v.m.cols, v.m.dtype, out));
+  if (v.lazy == 2) {  // the root-mean-square norm: no mean, no shift
+    KERNEL(k_rmsnorm, ctx, out->p, v.x, v.ldx, nullptr, v.gamma, v.eps, out->rows, out->cols, out->dtype, ctx->stream);
+    return 0;
+  }
   return layernorm(ctx, *out, v.x, v.gamma, v.beta, v.eps, nullptr);
 }
 
@@ -581,14 +586,19 @@ struct PyPosition : Position {
 
 struct PyMixer : Mixer {
   int id;
-  PyMixer(int i, int flags) : id(i) { accepts_lazy = false, wants_state = (flags & ENG_WANTS_STATE) != 0; }
+  PyMixer(int i, int flags) : id(i) {
+    accepts_lazy = (flags & ENG_ACCEPTS_LAZY) != 0, wants_state = (flags & ENG_WANTS_STATE) != 0;
+  }
   int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes) override {
     return forward_with_state(ctx, x, residual, slot, writes, -1);
   }
   int forward_with_state(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes,
                          int state_slot) override {
     EngCall c = {};
-    TRY(materialize(ctx, x, &c.x));
+    if (x.lazy && accepts_lazy && !x.packed)
+      c.x = x.m, c.x_lazy = x;  // (its first product norms the rows itself, or its Python side asks for them)
+    else
+      TRY(materialize(ctx, x, &c.x));
     c.residual = residual, c.cache_slot = slot, c.writes_cache = writes, c.state_slot = state_slot;
     return call_python(id, ENG_CB_MIXER, ctx, &c);
   }
@@ -596,10 +606,13 @@ struct PyMixer : Mixer {
 
 struct PyFeedForward : FeedForward {
   int id;
-  PyFeedForward(int i, int flags) : id(i) { accepts_lazy = false, (void)flags; }
+  PyFeedForward(int i, int flags) : id(i) { accepts_lazy = (flags & ENG_ACCEPTS_LAZY) != 0; }
   int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual) override {
     EngCall c = {};
-    TRY(materialize(ctx, x, &c.x));
+    if (x.lazy && accepts_lazy && !x.packed)
+      c.x = x.m, c.x_lazy = x;
+    else
+      TRY(materialize(ctx, x, &c.x));
     c.residual = residual;
     return call_python(id, ENG_CB_FFN, ctx, &c);
   }

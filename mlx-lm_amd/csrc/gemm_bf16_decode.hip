@@ -251,7 +251,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
       const int gk = min(tid * 4, p.K - 4);  // K / 4 <= 512 pieces: one a thread, surplus threads repeat the last
       if (first) {
         g4 = *(const float4*)(p.gamma + gk);
-        b4 = *(const float4*)(p.beta + gk);
+        b4 = p.beta ? *(const float4*)(p.beta + gk) : make_float4(0.f, 0.f, 0.f, 0.f);
         asm volatile("" ::: "memory");  // keep the weights' loads behind these
         __builtin_amdgcn_sched_barrier(0);
         load_pass(w0, 0);
@@ -262,7 +262,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
         if ((lane + 64 * i) * 4 >= p.K) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
       }
-      const float mean = wave_sum(s) / (float)p.K;
+      // (no shift: the root-mean-square norm, which takes no mean off either)
+      const float mean = p.beta ? wave_sum(s) / (float)p.K : 0.f;
       float q = 0.f;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
@@ -823,8 +824,9 @@ extern "C" int gemm_bf16_decode(
   if (!aligned16(W)) FAIL("gemm_bf16_decode: W must be 16-byte aligned");
   if (A && (lda % 8 != 0 || lda < K || !aligned16(A))) FAIL("gemm_bf16_decode: A rows must be 16-byte aligned");
   if (X && (ldx % 4 != 0 || ldx < K || !aligned16(X))) FAIL("gemm_bf16_decode: X rows must be 16-byte aligned");
-  if (X && (!gamma || !beta || !aligned16(gamma) || !aligned16(beta)))
-    FAIL("gemm_bf16_decode: the norm needs scale and shift, 16-byte aligned");
+  // (beta null: x / sqrt(mean(x^2) + eps) * gamma instead of the LayerNorm)
+  if (X && (!gamma || !aligned16(gamma) || !aligned16(beta)))
+    FAIL("gemm_bf16_decode: the norm needs a scale (and a shift, or none), 16-byte aligned");
   DecodeGemmArgs p;
   if (fill_epilogue(p, "gemm_bf16_decode", out, bias, M, N, ldo, flags, k_pages, v_pages, page_stride,
                     block_table, max_blocks, token_req, positions, q_width, kv_width, head_dim, page_size))

@@ -102,10 +102,17 @@ struct RmsNorm : Norm {
   float eps;
   const float* gamma;
   RmsNorm(int w, float e, const float* g) : width(w), eps(e), gamma(g) {}
-  int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool, const EngWeight*, bool,
+  int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool lazy, const EngWeight*, bool,
               EngValue* out) override {
     if (x.cols != width || x.dtype != DT_F32) return host->fail("rmsnorm: float32 rows of width %d", width);
     *out = EngValue{};
+    if (lazy && !rows) {
+      // the consumer's first matrix product may norm the rows itself (lazy 2: no mean, no shift)
+      out->lazy = 2, out->x = (const float*)x.p, out->ldx = x.ld, out->gamma = gamma, out->beta = nullptr;
+      out->eps = eps;
+      out->m = EngMat{nullptr, x.rows, width, width, ctx->dtype};
+      return 0;
+    }
     if (host->take(ctx, rows ? n_rows : x.rows, width, ctx->dtype, &out->m)) return 1;
     if (rmsnorm(out->m.p, (const float*)x.p, x.ld, rows, gamma, eps, out->m.rows, width, ctx->dtype, ctx->stream))
       return host->fail("%s", g_err);

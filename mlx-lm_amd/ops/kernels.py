@@ -164,23 +164,45 @@ def layernorm(out, x, gamma, beta, eps, rows=None):
 
 
 class NormedInput:
-    """The LayerNorm of float32 rows, not computed yet.
+    """The LayerNorm of float32 rows (``rms``: their root-mean-square norm, no mean taken off and
+    no shift), not computed yet.
 
     ``linear`` takes it as its input and, where its kernel can, norms the rows
     itself while the first weights are on their way; anything else calls
     ``materialize()`` and gets the tensor.
     """
 
-    def __init__(self, alloc, x, gamma, beta, eps, dtype):
+    def __init__(self, alloc, x, gamma, beta, eps, dtype, rms=False):
         self.alloc, self.x, self.gamma, self.beta, self.eps, self.dtype = alloc, x, gamma, beta, eps, dtype
+        self.rms = bool(rms)
         self.shape = tuple(x.shape)
         self._out = None
 
     def materialize(self):
         if self._out is None:
             self._out = self.alloc(self.shape, self.dtype)
-            layernorm(self._out, self.x, self.gamma, self.beta, self.eps)
+            if self.rms:
+                rmsnorm(self._out, self.x, self.gamma, self.eps)
+            else:
+                layernorm(self._out, self.x, self.gamma, self.beta, self.eps)
         return self._out
+
+
+def normed(x):
+    """``x`` as a tensor: a ``NormedInput`` is computed (once), a tensor is itself."""
+    return x.materialize() if isinstance(x, NormedInput) else x
+
+
+def rmsnorm(out, x, weight, eps):
+    """``out = x / sqrt(mean(x^2) + eps) * weight`` over float32 rows ``x``; ``out`` float32 or bfloat16."""
+    lib = build.load("rmsnorm")
+    ldx = _f32_rows(x, "x", out.shape[1])
+    _dev(weight, "weight", torch.float32)
+    _need(out.is_contiguous() and out.dtype in DT and weight.numel() == out.shape[1] and x.shape[0] >= out.shape[0], "rmsnorm: shapes")
+    rc = lib.rmsnorm(_ptr(out), _ptr(x), _c_int(ldx), None, _ptr(weight), _c_float(eps), _c_int(out.shape[0]),
+                     _c_int(out.shape[1]), _c_int(DT[out.dtype]), _stream())
+    build.check(lib, rc, "rmsnorm")
+    return out
 
 
 class KVScatter:
@@ -482,7 +504,7 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
             a = a.materialize()
     if isinstance(a, NormedInput):
         _dev(a.x, "x", torch.float32)
-        call.a.lazy, call.a.ldx = 1, a.x.stride(0)
+        call.a.lazy, call.a.ldx = 2 if a.rms else 1, a.x.stride(0)
         call.a.m = native.EngMat(None, a.shape[0], a.shape[1], a.shape[1], DT[a.dtype])
         call.a.x, call.a.gamma, call.a.beta, call.a.eps = a.x.data_ptr(), native.ptr(a.gamma), native.ptr(a.beta), a.eps
     elif isinstance(a, PackedRows):

@@ -22,6 +22,7 @@ MAX_GROUPS = 16
 
 DT = {torch.float32: 0, torch.bfloat16: 1, torch.int32: 2}
 TORCH_DT = {0: torch.float32, 1: torch.bfloat16, 2: torch.int32}
+DT_F32 = 0
 
 # kinds of part and callback methods (csrc/engine.h)
 NORM, MIXER, FFN, BLOCK, POSITION, EMBEDDING, HEAD, MODEL = range(1, 9)
@@ -82,7 +83,8 @@ class EngCtx(Structure):
 class EngCall(Structure):
     _fields_ = [("x", EngMat), ("residual", EngMat), ("out", EngMat), ("q", EngMat), ("k", EngMat),
                 ("rows", c_void_p), ("n_rows", c_int), ("cache_slot", c_int), ("writes_cache", c_int),
-                ("lazy", c_int), ("state_slot", c_int), ("pad_", c_int), ("result", EngMat), ("index", c_void_p), ("nbytes", c_size_t)]
+                ("lazy", c_int), ("state_slot", c_int), ("pad_", c_int), ("result", EngMat), ("index", c_void_p), ("nbytes", c_size_t),
+                ("x_lazy", EngValue)]
 
 
 class EngScatter(Structure):
@@ -295,17 +297,32 @@ def array_ids(key, names):
     return base
 
 
+def _input_of(ctx, call):
+    """A mixer's or feed-forward's input: a tensor, or, for a part that asked for it, the norm that
+    is not computed yet (``kernels.NormedInput``)."""
+    v = call.x_lazy
+    if not v.lazy:
+        return ctx.tensor(call.x)
+    from . import kernels
+
+    rows, width = call.x.rows, call.x.cols
+    x = ctx.tensor(EngMat(v.x, rows, width, v.ldx, DT_F32))
+    gamma = ctx.tensor(EngMat(v.gamma, 1, width, width, DT_F32))[0]
+    beta = ctx.tensor(EngMat(v.beta, 1, width, width, DT_F32))[0] if v.beta else None
+    return kernels.NormedInput(ctx.scratch, x, gamma, beta, v.eps, TORCH_DT[call.x.dtype], rms=v.lazy == 2)
+
+
 def run_python_part(part, method, ctx, call):
     """A callback part's turn: build tensors over the native side's matrices, call the method."""
     T = ctx.tensor
     if method == CB_MIXER:
         if call.state_slot >= 0 and getattr(part, "wants_state", False):
-            part.forward(ctx, T(call.x), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache),
+            part.forward(ctx, _input_of(ctx, call), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache),
                          state=ctx.cache_view(call.state_slot))
         else:
-            part.forward(ctx, T(call.x), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache))
+            part.forward(ctx, _input_of(ctx, call), T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache))
     elif method == CB_FFN:
-        part.forward(ctx, T(call.x), T(call.residual))
+        part.forward(ctx, _input_of(ctx, call), T(call.residual))
     elif method == CB_BLOCK:
         if call.state_slot >= 0:
             part.forward(ctx, T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache),

@@ -79,6 +79,9 @@ class Part:
             flags |= native.SETTLES_PENDING
         if getattr(self, "wants_state", False):
             flags |= native.WANTS_STATE
+        if getattr(self, "takes_normed_input", False):
+            # (a mixer or feed-forward whose ``x`` may be a ``kernels.NormedInput``: its first product norms the rows)
+            flags |= native.ACCEPTS_LAZY
         self._python_id = native.register_python_part(self)
         return native.made(native.lib().eng_make_callback(self.native_kind, self._python_id, flags),
                            type(self).__name__)

@@ -127,6 +127,7 @@ class GatedMLP(FeedForward):
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
+    takes_normed_input = True  # ``x`` may be a ``kernels.NormedInput``: the first product norms the rows itself
 
     def __init__(self, width, inner, gate_name="gate", up_name="up", down_name="down", prefix=""):
         super().__init__(prefix)

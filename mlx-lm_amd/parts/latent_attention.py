@@ -32,6 +32,7 @@ class LatentAttention(Mixer):
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
+    takes_normed_input = True  # ``x`` may be a ``kernels.NormedInput``: the first product norms the rows itself
     step_arrays_key = CausalSelfAttention.step_arrays_key
     step_array_names = CausalSelfAttention.step_array_names
     step_arrays = staticmethod(CausalSelfAttention.step_arrays)
