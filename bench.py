@@ -117,10 +117,10 @@ def zatinex_config(s):
     second such layer reads the first one's latents.  A gated feed-forward of two thirds of GPT-2's
     inner size (three matrices where GPT-2 has two)."""
     H, d, D = s["heads"], s["dim"], s["width"]
-    scaling = {"factor": 4.0, "original": 512, "fast": 32.0, "slow": 1.0}
-    attention = {"type": "attention", "mixer": {"heads": H // 2, "kv_heads": H // 2, "dim": d, "vdim": 2 * d, "conv": 4, "diff": 0.5,
+    scaling = {"factor": 8.0, "original": 1024, "fast": 16.0, "slow": 2.0}
+    attention = {"type": "attention", "mixer": {"heads": H // 2, "kv_heads": H // 2, "dim": d, "vdim": 2 * d, "conv": 4, "diff": 0.3,
                                                 "scale": d ** -0.5, "rot": {"dims": d, "base": 10000.0, "scaling": scaling}}}
-    gla = {"type": "gla", "mixer": {"heads": H, "dim": d, "vdim": d, "tau": 16.0}}
+    gla = {"type": "gla", "mixer": {"heads": H, "dim": d, "vdim": d, "tau": 8.0}}
     latent = {"heads": H, "dim": d, "rot_dim": d // 2, "vdim": d, "q_rank": D // 2, "kv_rank": 192,
               "scale": (d + d // 2) ** -0.5, "rot": {"dims": d // 2, "base": 10000.0}}
     mlp = {"kind": "dense", "ff": s["ff"] * 2 // 3 // 64 * 64}

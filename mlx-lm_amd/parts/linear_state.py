@@ -148,13 +148,16 @@ class GatedLinearAttention(_SequenceArrays, Mixer):
     middle, laid out like the keys.  Each head's ``o`` is RMS-normed over ``value_dim`` with one
     weight for all heads, the heads are multiplied by ``silu(Wg x)`` and projected by ``Wo``.
     ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start) is the request's
-    state.  One product gives ``[q | k | v | g]`` as float32 rows; ``z`` is a float32 row; the
+    state.  One product gives ``[q | k | v | g | z]`` as float32 rows (``Wa2 Wa1`` is multiplied
+    out when the weights are loaded: one product and no launches for the middle, for ``key_dim *
+    n_heads`` more rows of weights); the
     logarithm of the decay (``log sigmoid(z) / tau``), the recurrence, the norm and the gate are
     32-bit (csrc/linear_state.hip; the factor of the queries rides on the keys, which gives the
     same outputs).  No counterpart in mlx_lm/models/gpt2.py.
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
+    takes_normed_input = True  # ``x`` may be a ``kernels.NormedInput``: the first product norms the rows itself
 
     def __init__(self, width, n_heads, key_dim, value_dim, tau, eps, decay_rank, prefix=""):
         super().__init__(prefix)
@@ -185,25 +188,23 @@ class GatedLinearAttention(_SequenceArrays, Mixer):
 
     def load(self, tensors):
         n = self._name
-        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in ("q", "k", "v", "g")]))
+        a1, a2 = tensors[n("a1")], tensors[n("a2")]
+        # the decay's two products through the narrow middle are one matrix times x: it rides in the
+        # projection beside q, k, v and g (made in float64, rounded once), its bias with it
+        decay_w = (a2.double() @ a1.double()).to(a1.dtype)
+        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in ("q", "k", "v", "g")] + [decay_w]))
+        self.in_b = torch.cat([tensors[n("a2.b")].new_zeros(2 * self.qk_width + 2 * self.v_width), tensors[n("a2.b")]]).contiguous()
         self.first_weight = self.in_w
-        a1 = tensors[n("a1")]
-        pad = -a1.shape[0] % 8  # (the middle is the second product's inner size: zero rows here meet zero columns there)
-        self.a1_w = _matrix(torch.cat([a1, a1.new_zeros(pad, a1.shape[1])]) if pad else a1)
-        self.a2_w, self.a2_b = _matrix(_padded_columns(tensors[n("a2")])), tensors[n("a2.b")]
         self.out_w = _matrix(_padded_columns(tensors[n("o")]))
         self.norm_w = tensors[n("norm")]
 
     def forward(self, ctx, x, residual, cache, writes_cache=True):
         T = x.shape[0]
         mark = ctx.scratch_mark()
-        u = ctx.scratch((T, 2 * self.qk_width + 2 * self.v_width), torch.float32)
-        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
-        mid = ctx.scratch((T, -(-self.decay_rank // 8) * 8), ctx.dtype)
-        kernels.linear(mid, x, self.a1_w, splits=kernels.splits_alone(T))
-        z = ctx.scratch((T, self.qk_width), torch.float32)
-        kernels.linear(z, mid, self.a2_w, bias=self.a2_b, splits=kernels.splits_alone(T))
+        u = ctx.scratch((T, 3 * self.qk_width + 2 * self.v_width), torch.float32)
+        kernels.linear(u, x, self.in_w, bias=self.in_b, splits=kernels.splits_alone(T))
         a, b = self.qk_width, 2 * self.qk_width
+        z = u[:, b + 2 * self.v_width:]
         out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
         kernels.state_scan(out, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, 0,
                            ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,

@@ -40,10 +40,10 @@ CONFIGS = {
         eps=1e-3),
     # wider, for bfloat16: heads of 64
     "C": _config(128, 300, [
-        _with_ff(_attention(4, 2, 64, 64, conv=3, rot={"dims": 32, "base": 1e4, "scaling": YARN}, diff=0.5), 96),
+        _with_ff(_attention(4, 2, 64, 64, conv=3, rot={"dims": 32, "base": 1e4, "scaling": YARN}, diff=0.45), 96),
         _gla(2, 64, 64, 8.0),
         _with_ff(_latent(4, 32, 16, 48, 48, 64, base=1e5), 96),
-        _with_ff(_gla(4, 32, 32, 16.0), 64),
+        _with_ff(_gla(4, 32, 32, 12.0), 64),
         _with_ff(_latent(2, 64, 16, 64, 32, 64, base=1e5, kv_from=2), 64)]),
 }
 SEEDS = {"A": 3, "B": 4, "C": 5}
