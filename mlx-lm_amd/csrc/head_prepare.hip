@@ -2,18 +2,22 @@
 // between the attention and the output projection, for mixers that shape their heads in ways of
 // their own.  Everything is 32-bit inside; the sources are the projections' float rows.
 //
-//   causal_conv     y[t, c] = act(b[c] + sum_j w[c, j] u[t - taps + 1 + j, c]) over a request's own
-//                   tokens; inputs of earlier steps come from the request's state row ([taps - 1, C],
-//                   the latest last, zero at a request's start), which conv_state_update
-//                   (linear_state.hip) brings up to date afterwards.  With `single` (every request
-//                   brings one token) the kernel moves the state up itself.
-//   head_prepare    a wave a (row, head): the head's `dim` columns from a float row; RMS norm over
+//   (causal convolution)  y[t, c] = sum_j w[c, j] u[t - taps + 1 + j, c] over a request's own tokens;
+//                   inputs of earlier steps come from the request's state row ([taps - 1, C], the
+//                   latest last, zero at a request's start), which conv_state_update
+//                   (linear_state.hip) brings up to date afterwards.  With `conv_single` (every
+//                   request brings one token) the kernel moves the state up itself.  It is an
+//                   option of head_prepare: the source's columns pass through it on their way in.
+//   head_prepare    a wave a (row, head): the head's `dim` columns from a float row (through the
+//                   convolution, where one is given); RMS norm over
 //                   the first `norm_dim` of them (times a weight of norm_dim values shared by all
 //                   heads, or none); rotation of the `rot_dims` columns from `rot_off` on by
 //                   position * inv_freq[i], pairs (2i, 2i + 1) or (i, i + rot_dims / 2), cos and
 //                   sin times `rot_mult`; then the head goes to `copies` places: copy c of head h
 //                   to column dst_head[c * n_heads + h] * dst_stride of the output row (h itself
-//                   without a table), zeros from `dim` up to `dst_fill` columns.
+//                   without a table), zeros from `dim` up to `dst_fill` columns.  The output is
+//                   rows of a matrix, or (block_table given) the pages of a cache: the row's
+//                   request and position say which page and place, as kv_write has it.
 //                   head_prepare_many: up to four such preparations in one launch.
 //   diff_combine    o = a1 - lambda a2 per head, where a1 and a2 are two heads of an attention's
 //                   output (tables say which), divided by its root mean square and multiplied by
@@ -23,30 +27,7 @@
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-// Thread (token row, channel).
-__global__ __launch_bounds__(256) void causal_conv_kernel(const float* __restrict__ u, int ldu, int col,
-                                                          const float* __restrict__ w, const float* __restrict__ b,
-                                                          int taps, int C, int act, float* __restrict__ state,
-                                                          size_t state_stride, size_t conv_offset,
-                                                          const int* __restrict__ token_req,
-                                                          const int* __restrict__ seq_start,
-                                                          const int* __restrict__ slot_ids, float* __restrict__ y,
-                                                          int ldy, int single) {
-  const int c = blockIdx.y * 256 + threadIdx.x, row = blockIdx.x;
-  if (c >= C) return;
-  const int req = token_req[row], local = row - seq_start[req];
-  float* old = state + (size_t)slot_ids[req] * state_stride + conv_offset;  // [taps - 1, C], the latest last
-  float acc = b ? b[c] : 0.f;
-  for (int j = taps - 1; j >= 0; --j) {  // the oldest input first
-    const int at = local - j;
-    const float in = at >= 0 ? u[(size_t)(row - j) * ldu + col + c] : old[(size_t)(taps - 1 + at) * C + c];
-    acc += w[(size_t)c * taps + (taps - 1 - j)] * in;
-    // every request brings one token: this thread alone reads and writes its request's inputs
-    // of channel c, so it moves them up by one as it goes (the oldest first)
-    if (single && j < taps - 1) old[(size_t)(taps - 2 - j) * C + c] = in;
-  }
-  y[(size_t)row * ldy + c] = act ? silu_f(acc) : acc;
-}
+#define PREPARE_CONV_MAX_DIM 256  // the widest head that passes a convolution
 
 struct PrepareArgs {
   const float* src;
@@ -62,26 +43,72 @@ struct PrepareArgs {
   void* dst;
   int ldd, dst_stride, dst_fill, copies;
   const int* dst_head;  // [copies, n_heads] or null
+  // a causal convolution over the source's columns (column c of the row is channel c), or conv_w null
+  const float* conv_w;  // [channels, taps]
+  int taps, conv_channels, conv_single;
+  float* conv_state;  // a request's row: [taps - 1, channels] at conv_offset, the latest last
+  size_t conv_state_stride, conv_offset;
+  const int* seq_start;  // [requests] the first row of a request in this step
+  const int* slot_ids;   // [requests] its state row
+  const int* token_req;  // [rows] (the convolution and the pages need it)
+  // dst is a cache's pages (of dst_stride columns a head) where block_table is given
+  const int* block_table;
+  int max_blocks, page_size;
+  size_t page_stride;
 };
 
 template <typename T>
 __device__ __forceinline__ void prepare_head(const PrepareArgs& a, long item, int lane) {
   if (item >= (long)a.n_rows * a.n_heads) return;  // whole waves leave; no barrier follows
   const int row = (int)(item / a.n_heads), h = (int)(item % a.n_heads);
-  const float* s = a.src + (size_t)row * a.lds + a.src_col + (size_t)h * a.src_stride;
+  const int first_col = a.src_col + h * a.src_stride;
+  const float* s = a.src + (size_t)row * a.lds + first_col;
+  const int req = (a.conv_w || a.block_table) ? a.token_req[row] : 0;
+  const int local = a.conv_w ? row - a.seq_start[req] : 0;  // the row's place among its request's rows of this step
+  float* old = a.conv_w ? a.conv_state + (size_t)a.slot_ids[req] * a.conv_state_stride + a.conv_offset : nullptr;
+  // column c of the head as the rest sees it: as it is, or through the convolution (the oldest
+  // input first), which is run once a column into the wave's own piece of LDS (the norm, the
+  // column's own turn and its partner's read it)
+  __shared__ float convolved[4][PREPARE_CONV_MAX_DIM];
+  float* cv = convolved[threadIdx.x >> 6];
+  if (a.conv_w) {
+    for (int c = lane; c < a.dim; c += 64) {
+      const int ch = first_col + c;
+      float acc = 0.f;
+      for (int j = a.taps - 1; j >= 0; --j) {
+        const int at = local - j;
+        const float u = at >= 0 ? s[c - (long)j * a.lds] : old[(size_t)(a.taps - 1 + at) * a.conv_channels + ch];
+        acc += a.conv_w[(size_t)ch * a.taps + (a.taps - 1 - j)] * u;
+      }
+      cv[c] = acc;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // (the wave's lanes read each other's columns)
+    __builtin_amdgcn_wave_barrier();
+  }
+  auto in = [&](int c) { return a.conv_w ? cv[c] : s[c]; };
   float rstd = 1.f;
   if (a.norm_dim > 0) {
     float q = 0.f;
-    for (int k = lane; k < a.norm_dim; k += 64) q += s[k] * s[k];
+    for (int k = lane; k < a.norm_dim; k += 64) {
+      const float u = in(k);
+      q += u * u;
+    }
     rstd = 1.0f / sqrtf(wave_sum(q) / (float)a.norm_dim + a.eps);
   }
-  const float pos = a.rot_dims ? (float)a.positions[row] : 0.f;
+  const int position = (a.rot_dims || a.block_table) ? a.positions[row] : 0;
+  const float pos = (float)position;
   const int half = a.rot_dims / 2;
+  // where head dh of this row starts in dst
+  const size_t page_base = a.block_table ? (size_t)a.block_table[(size_t)req * a.max_blocks + position / a.page_size] * a.page_stride : 0;
+  auto head_at = [&](int dh) {
+    return a.block_table ? page_base + ((size_t)dh * a.page_size + position % a.page_size) * a.dst_stride
+                         : (size_t)row * a.ldd + (size_t)dh * a.dst_stride;
+  };
   for (int k = lane; k < a.dst_fill; k += 64) {
     float v = 0.f;
     if (k < a.dim) {
       const int rel = k - a.rot_off;
-      auto at = [&](int c) { return c < a.norm_dim ? s[c] * rstd * (a.norm_w ? a.norm_w[c] : 1.f) : s[c]; };
+      auto at = [&](int c) { return c < a.norm_dim ? in(c) * rstd * (a.norm_w ? a.norm_w[c] : 1.f) : in(c); };
       v = at(k);
       if (rel >= 0 && rel < a.rot_dims) {
         int i, partner;
@@ -99,7 +126,18 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& a, long item, in
     }
     for (int c = 0; c < a.copies; ++c) {
       const int dh = a.dst_head ? a.dst_head[c * a.n_heads + h] : h;
-      ((T*)a.dst)[(size_t)row * a.ldd + (size_t)dh * a.dst_stride + k] = from_f32<T>(v);
+      ((T*)a.dst)[head_at(dh) + k] = from_f32<T>(v);
+    }
+  }
+  if (a.conv_w && a.conv_single && a.taps > 1) {
+    // every request brings one token: this wave alone reads and writes its request's inputs of this
+    // head's channels, so it moves them up by one itself, after everything above has been read
+    // (a lane read its neighbours' channels for the rotation: the wave's loads are waited for first)
+    __builtin_amdgcn_s_waitcnt(0);
+    for (int k = lane; k < a.dim; k += 64) {
+      const int ch = first_col + k;
+      for (int j = 0; j + 2 < a.taps; ++j) old[(size_t)j * a.conv_channels + ch] = old[(size_t)(j + 1) * a.conv_channels + ch];
+      old[(size_t)(a.taps - 2) * a.conv_channels + ch] = s[k];
     }
   }
 }
@@ -162,21 +200,6 @@ __global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ x, int l
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
-extern "C" int causal_conv(const float* u, int ldu, int col, const float* w, const float* b, int taps, int C, int act,
-                           float* state, size_t state_stride, size_t conv_offset, const int* token_req,
-                           const int* seq_start, const int* slot_ids, float* y, int ldy, int n_tokens, int single,
-                           hipStream_t stream) {
-  if (n_tokens <= 0) return 0;
-  if (!u || !w || !state || !token_req || !seq_start || !slot_ids || !y) FAIL("causal_conv: null pointer");
-  if (taps < 1 || C <= 0 || col < 0 || col + C > ldu || ldy < C)
-    FAIL("causal_conv: %d taps, %d channels from column %d, rows of %d and %d", taps, C, col, ldu, ldy);
-  dim3 grid(n_tokens, (C + 255) / 256), block(256);
-  hipLaunchKernelGGL(causal_conv_kernel, grid, block, 0, stream, u, ldu, col, w, b, taps, C, act, state, state_stride,
-                     conv_offset, token_req, seq_start, slot_ids, y, ldy, single);
-  CHECK_LAUNCH("causal_conv");
-  return 0;
-}
-
 static int prepare_args_fit(const PrepareArgs& a) {
   if (!a.src || !a.dst) FAIL("head_prepare: null pointer");
   if (a.dim <= 0 || a.src_col < 0 || a.src_col + (long)(a.n_heads - 1) * a.src_stride + a.dim > a.lds)
@@ -187,8 +210,14 @@ static int prepare_args_fit(const PrepareArgs& a) {
     FAIL("head_prepare: %d turning columns from %d in a head of %d", a.rot_dims, a.rot_off, a.dim);
   if (a.copies < 1 || a.dst_fill < a.dim || a.dst_fill > a.dst_stride)
     FAIL("head_prepare: %d copies, %d columns filled of %d, a head of %d", a.copies, a.dst_fill, a.dst_stride, a.dim);
-  if (!a.dst_head && (a.copies != 1 || (long)(a.n_heads - 1) * a.dst_stride + a.dst_fill > a.ldd))
+  if (!a.block_table && !a.dst_head && (a.copies != 1 || (long)(a.n_heads - 1) * a.dst_stride + a.dst_fill > a.ldd))
     FAIL("head_prepare: the heads do not fit rows of %d", a.ldd);
+  if (a.conv_w && a.dim > PREPARE_CONV_MAX_DIM) FAIL("head_prepare: heads of %d columns through a convolution (at most %d)", a.dim, PREPARE_CONV_MAX_DIM);
+  if (a.conv_w && (a.taps < 1 || a.conv_channels < a.src_col + (a.n_heads - 1) * a.src_stride + a.dim || !a.conv_state ||
+                   !a.seq_start || !a.slot_ids || !a.token_req))
+    FAIL("head_prepare: a convolution of %d taps over %d channels needs its state and the rows' requests", a.taps, a.conv_channels);
+  if (a.block_table && (!a.token_req || !a.positions || a.max_blocks <= 0 || a.page_size <= 0 || a.dst_fill != a.dst_stride))
+    FAIL("head_prepare: pages of %d places need the rows' requests and positions, and whole heads of %d columns", a.page_size, a.dst_stride);
   return 0;
 }
 

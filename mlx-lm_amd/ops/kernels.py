@@ -1034,31 +1034,6 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
 # between a projection and the attention that reads its heads, and behind it (csrc/head_prepare.hip)
 
 
-def causal_conv(y, u, col, weight, bias, state, conv_offset, token_req, seq_start, slot_ids, silu=False, single_tokens=False):
-    """``y[t, c] = act(bias[c] + sum_j weight[c, j] * u[t - taps + 1 + j, col + c])`` over each request's own
-    tokens; the inputs of earlier steps come from the request's row of ``state`` (``[taps - 1,
-    channels]`` at ``conv_offset``, the latest last; ``conv_state_update`` brings it up to date
-    afterwards, or this kernel itself with ``single_tokens``, when every request brings one token).
-    ``u`` and ``y`` are float32 rows."""
-    lib = build.load("head_prepare")
-    C, taps = weight.shape
-    ldu, ldy = _f32_rows(u, "u", col + C), _f32_rows(y, "y", C)
-    _dev(weight, "weight", torch.float32)
-    _dev(state, "state", torch.float32)
-    _need(weight.is_contiguous() and (bias is None or bias.numel() == C), "causal_conv: weight [channels, taps], bias [channels]")
-    _need(state.dim() == 2 and conv_offset + (taps - 1) * C <= state.shape[1], "causal_conv: the state rows are too short")
-    for name, t in (("token_req", token_req), ("seq_start", seq_start), ("slot_ids", slot_ids)):
-        _dev(t, name, torch.int32)
-    T = y.shape[0]
-    _need(u.shape[0] >= T and token_req.numel() >= T, "causal_conv: fewer input rows than output rows")
-    rc = lib.causal_conv(_ptr(u), _c_int(ldu), _c_int(col), _ptr(weight), _ptr(bias), _c_int(taps), _c_int(C),
-                         _c_int(int(bool(silu))), _ptr(state), _c_size_t(state.stride(0)), _c_size_t(conv_offset),
-                         _ptr(token_req), _ptr(seq_start), _ptr(slot_ids), _ptr(y), _c_int(ldy), _c_int(T),
-                         _c_int(int(bool(single_tokens))), _stream())
-    build.check(lib, rc, "causal_conv")
-    return y
-
-
 class PrepareArgs(ctypes.Structure):
     """Mirror of ``PrepareArgs`` in csrc/head_prepare.hip."""
 
@@ -1066,7 +1041,43 @@ class PrepareArgs(ctypes.Structure):
                 ("n_heads", _c_int), ("dim", _c_int), ("norm_dim", _c_int), ("norm_w", _vp), ("eps", _c_float),
                 ("rot_off", _c_int), ("rot_dims", _c_int), ("interleaved", _c_int), ("inv_freq", _vp),
                 ("rot_mult", _c_float), ("positions", _vp), ("dst", _vp), ("ldd", _c_int), ("dst_stride", _c_int),
-                ("dst_fill", _c_int), ("copies", _c_int), ("dst_head", _vp)]
+                ("dst_fill", _c_int), ("copies", _c_int), ("dst_head", _vp),
+                ("conv_w", _vp), ("taps", _c_int), ("conv_channels", _c_int), ("conv_single", _c_int), ("conv_state", _vp),
+                ("conv_state_stride", _c_size_t), ("conv_offset", _c_size_t), ("seq_start", _vp), ("slot_ids", _vp),
+                ("token_req", _vp), ("block_table", _vp), ("max_blocks", _c_int), ("page_size", _c_int),
+                ("page_stride", _c_size_t)]
+
+
+class ConvolutionAhead:
+    """A causal convolution that ``head_prepare`` runs over its source's columns on their way in:
+    ``y[t, c] = sum_j weight[c, j] * u[t - taps + 1 + j, c]`` over each request's own tokens (column
+    ``c`` of ``u`` is channel ``c``); the inputs of earlier steps come from the request's row of
+    ``state`` (``[taps - 1, channels]`` at ``offset``, the latest last).  With ``single`` (every
+    request brings one token) the kernel also moves these up by one; otherwise ``conv_state_update``
+    does afterwards."""
+
+    def __init__(self, weight, state, offset, token_req, seq_start, slot_ids, single):
+        _dev(weight, "weight", torch.float32)
+        _dev(state, "state", torch.float32)
+        for name, t in (("token_req", token_req), ("seq_start", seq_start), ("slot_ids", slot_ids)):
+            _dev(t, name, torch.int32)
+        channels, taps = weight.shape
+        _need(weight.is_contiguous() and state.dim() == 2 and offset + (taps - 1) * channels <= state.shape[1],
+              "a convolution's weight is [channels, taps] and its state rows hold taps - 1 inputs of every channel")
+        self.weight, self.state, self.offset, self.single = weight, state, int(offset), bool(single)
+        self.token_req, self.seq_start, self.slot_ids = token_req, seq_start, slot_ids
+
+
+class PagesOut:
+    """The keys' (or values') pages of a cache view as the place ``head_prepare`` writes to: a row goes
+    where its request's block table and its position say, as ``kv_write`` has it."""
+
+    def __init__(self, kv, values, block_table, token_req, positions):
+        self.pages = kv.v if values else kv.k
+        self.kv, self.block_table, self.token_req, self.positions = kv, block_table, token_req, positions
+        for name, t in (("block_table", block_table), ("token_req", token_req), ("positions", positions)):
+            _dev(t, name, torch.int32)
+        self.dtype, self.shape = self.pages.dtype, None
 
 
 def head_prepare(dst, src, src_col, n_heads, dim, **options):
@@ -1076,7 +1087,8 @@ def head_prepare(dst, src, src_col, n_heads, dim, **options):
     by ``position * inv_freq[i]`` (pairs ``(2i, 2i + 1)`` with ``interleaved``, else ``(i, i +
     rot_dims / 2)``; cos and sin times ``rot_mult``); written to ``dst`` (float32 or bfloat16) at
     column ``dst_head[c, h] * dst_stride`` for each of ``copies`` copies (``h * dst_stride`` without
-    a table), with zeros from ``dim`` up to ``dst_fill`` columns."""
+    a table), with zeros from ``dim`` up to ``dst_fill`` columns.  ``conv`` (a ``ConvolutionAhead``):
+    the source's columns pass a causal convolution first.  ``dst`` may be a ``PagesOut``."""
     lib = build.load("head_prepare")
     a = _prepare_args(dst, src, src_col, n_heads, dim, **options)
     rc = lib.head_prepare(ctypes.byref(a), _c_int(DT[dst.dtype]), _stream())
@@ -1086,7 +1098,7 @@ def head_prepare(dst, src, src_col, n_heads, dim, **options):
 
 def head_prepare_many(*calls):
     """Several ``head_prepare`` calls in one launch: each of ``calls`` is ``(dst, src, src_col,
-    n_heads, dim, options)``; at most four, their ``dst`` of one dtype."""
+    n_heads, dim, options)``; at most four, their ``dst`` (a matrix or a ``PagesOut``) of one dtype."""
     lib = build.load("head_prepare")
     _need(1 <= len(calls) <= 4 and len({c[0].dtype for c in calls}) == 1, "head_prepare_many: one to four calls, outputs of one dtype")
     args = (PrepareArgs * len(calls))(*[_prepare_args(*c[:5], **c[5]) for c in calls])
@@ -1096,14 +1108,15 @@ def head_prepare_many(*calls):
 
 def _prepare_args(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=None, dst_fill=None, norm_dim=0,
                   norm_weight=None, eps=0.0, rot_off=0, rot_dims=0, inv_freq=None, rot_mult=1.0, interleaved=True,
-                  positions=None, dst_head=None, copies=1):
+                  positions=None, dst_head=None, copies=1, conv=None):
     a = PrepareArgs()
     src_stride = dim if src_stride is None else src_stride
+    n_rows = src.shape[0] if isinstance(dst, PagesOut) else dst.shape[0]
     dst_stride = dim if dst_stride is None else dst_stride
     a.lds = _f32_rows(src, "src", src_col + (n_heads - 1) * src_stride + dim)
     a.src, a.src_col, a.src_stride = src.data_ptr(), int(src_col), int(src_stride)
-    a.n_rows, a.n_heads, a.dim = dst.shape[0], int(n_heads), int(dim)
-    _need(src.shape[0] >= dst.shape[0], "head_prepare: fewer source rows than rows of dst")
+    a.n_rows, a.n_heads, a.dim = n_rows, int(n_heads), int(dim)
+    _need(src.shape[0] >= n_rows, "head_prepare: fewer source rows than rows of dst")
     a.norm_dim, a.eps = int(norm_dim), float(eps)
     if norm_weight is not None:
         _dev(norm_weight, "norm_weight", torch.float32)
@@ -1112,17 +1125,31 @@ def _prepare_args(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=N
     if rot_dims:
         _dev(inv_freq, "inv_freq", torch.float32)
         _dev(positions, "positions", torch.int32)
-        _need(inv_freq.numel() == rot_dims // 2 and positions.numel() >= dst.shape[0], "head_prepare: inv_freq / positions")
+        _need(inv_freq.numel() == rot_dims // 2 and positions.numel() >= n_rows, "head_prepare: inv_freq / positions")
         a.rot_off, a.rot_dims, a.interleaved = int(rot_off), int(rot_dims), int(bool(interleaved))
         a.inv_freq, a.rot_mult, a.positions = inv_freq.data_ptr(), float(rot_mult), positions.data_ptr()
-    a.ldd = _rows2d(dst, "dst")
     _need(dst.dtype in DT, "head_prepare: dst is float32 or bfloat16")
-    a.dst, a.dst_stride, a.dst_fill, a.copies = dst.data_ptr(), int(dst_stride), int(dst_fill or dim), int(copies)
+    a.dst_stride, a.dst_fill, a.copies = int(dst_stride), int(dst_fill or dim), int(copies)
     if dst_head is not None:
         _dev(dst_head, "dst_head", torch.int32)
         _need(dst_head.numel() == copies * n_heads, "head_prepare: dst_head is [copies, heads]")
         a.dst_head = dst_head.data_ptr()
-    _need(dst.shape[1] >= (n_heads * copies - 1) * dst_stride + a.dst_fill, "head_prepare: dst rows are too short for the heads")
+    if isinstance(dst, PagesOut):
+        kv = dst.kv
+        _need(kv.head_dim == dst_stride and n_heads * copies <= kv.n_kv_heads and dst.token_req.numel() >= n_rows
+              and dst.positions.numel() >= n_rows, "head_prepare: the heads do not fit the cache's pages")
+        a.dst, a.block_table, a.max_blocks = dst.pages.data_ptr(), dst.block_table.data_ptr(), dst.block_table.shape[1]
+        a.page_size, a.page_stride = kv.page_size, kv.page_stride
+        a.token_req, a.positions = dst.token_req.data_ptr(), dst.positions.data_ptr()
+    else:
+        a.ldd, a.dst = _rows2d(dst, "dst"), dst.data_ptr()
+        _need(dst.shape[1] >= (n_heads * copies - 1) * dst_stride + a.dst_fill, "head_prepare: dst rows are too short for the heads")
+    if conv is not None:
+        channels, taps = conv.weight.shape
+        _need(src.shape[1] >= channels and conv.token_req.numel() >= n_rows, "head_prepare: the convolution's channels are the source's columns")
+        a.conv_w, a.taps, a.conv_channels, a.conv_single = conv.weight.data_ptr(), taps, channels, int(conv.single)
+        a.conv_state, a.conv_state_stride, a.conv_offset = conv.state.data_ptr(), conv.state.stride(0), conv.offset
+        a.seq_start, a.slot_ids, a.token_req = conv.seq_start.data_ptr(), conv.slot_ids.data_ptr(), conv.token_req.data_ptr()
     return a
 
 

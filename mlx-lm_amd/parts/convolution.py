@@ -14,7 +14,8 @@ class ShortConvolution(_SequenceArrays, Part):
     (``state_need``) and zeroed when a request starts, which gives the zeros before its first token.
     Not a mixer: a mixer builds it, runs it between its projection and what follows, and lists it
     among its ``sub_parts`` so that the model hands it its tensors and its step arrays (where each
-    request's tokens start).  32-bit throughout (csrc/head_prepare.hip: ``causal_conv``).  No
+    request's tokens start).  32-bit throughout; it runs inside ``head_prepare`` as that reads the
+    projection's columns (csrc/head_prepare.hip).  No
     counterpart in mlx_lm/models/gpt2.py."""
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
@@ -42,15 +43,18 @@ class ShortConvolution(_SequenceArrays, Part):
     def state_need(self):
         return StateNeed((self.state_floats,), "float32") if self.state_floats else None
 
-    def forward(self, ctx, y, u, state, offset=0):
-        """``y`` from ``u`` (float32 rows of ``n_channels`` columns from column 0); ``state``: the
-        requests' state rows, this part's floats from ``offset`` on."""
+    def ahead(self, ctx, state, offset=0):
+        """What ``kernels.head_prepare`` takes as ``conv``: the convolution runs as the heads are read.
+        ``state``: the requests' state rows, this part's floats from ``offset`` on."""
         if not self.state_floats:
             state, offset = self.no_state, 0
-        starts = ctx.array("sequences.starts")
         single = ctx.array("sequences.longest") == 1
-        kernels.causal_conv(y, u, 0, self.weight, None, state, offset, ctx.token_req, starts, ctx.slot_ids,
-                            single_tokens=single)
-        if not single and self.taps > 1:
-            kernels.conv_state_update(u, 0, self.taps, self.n_channels, state, offset, starts, ctx.array("sequences.lens"),
-                                      ctx.slot_ids, ctx.n_requests)
+        return kernels.ConvolutionAhead(self.weight, state, offset, ctx.token_req, ctx.array("sequences.starts"), ctx.slot_ids, single)
+
+    def keep_inputs(self, ctx, u, state, offset=0):
+        """After the step's rows ``u`` (the convolution's inputs) have been read: the requests' last
+        ``taps - 1`` inputs for the next step (nothing to do where every request brought one token:
+        the kernel that read them moved them up itself)."""
+        if self.taps > 1 and ctx.array("sequences.longest") != 1:
+            kernels.conv_state_update(u, 0, self.taps, self.n_channels, state, offset, ctx.array("sequences.starts"),
+                                      ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests)

@@ -116,24 +116,21 @@ class DifferentialAttention(Mixer):
         mark = ctx.scratch_mark()
         u = ctx.scratch((T, self.q_cols + self.k_cols + self.v_cols), torch.float32)
         kernels.linear(u, x, self.in_w, bias=self.in_b, splits=kernels.splits_alone(T))
-        if self.conv is not None:
-            y = ctx.scratch(tuple(u.shape), torch.float32)
-            self.conv.forward(ctx, y, u, state.state if state is not None else None)
-            u = y
-        rot = dict(rot_dims=self.rot_dims, inv_freq=self.inv_freq, rot_mult=self.rot_mult, positions=ctx.positions)
+        conv = self.conv.ahead(ctx, state.state if state is not None else None) if self.conv is not None else None
+        rot = dict(rot_dims=self.rot_dims, inv_freq=self.inv_freq, rot_mult=self.rot_mult, positions=ctx.positions, conv=conv)
         q = ctx.scratch((T, H2 * hd), ctx.dtype)
         calls = [(q, u, 0, H2, d, dict(dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.q_norm, eps=self.eps,
                                        dst_head=self.q_place, **rot))]
         if writes_cache:
-            k = ctx.scratch((T, G2 * hd), ctx.dtype)
-            v = ctx.scratch((T, G2 * hd), ctx.dtype)
-            calls.append((k, u, self.q_cols, G2, d, dict(dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.k_norm,
-                                                         eps=self.eps, **rot)))
-            calls.append((v, u, self.q_cols + self.k_cols, self.n_kv_heads, self.value_dim,
-                          dict(dst_stride=hd, dst_fill=hd, dst_head=self.v_place, copies=2)))
-        kernels.head_prepare_many(*calls)  # (queries, keys and values in one launch)
-        if writes_cache:
-            kernels.kv_write(k, v, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
+            # keys and values go straight to their pages
+            pages = [kernels.PagesOut(cache.kv, values, cache.block_table, ctx.token_req, ctx.positions) for values in (False, True)]
+            calls.append((pages[0], u, self.q_cols, G2, d, dict(dst_stride=hd, dst_fill=hd, norm_dim=d, norm_weight=self.k_norm,
+                                                                eps=self.eps, **rot)))
+            calls.append((pages[1], u, self.q_cols + self.k_cols, self.n_kv_heads, self.value_dim,
+                          dict(dst_stride=hd, dst_fill=hd, dst_head=self.v_place, copies=2, conv=conv)))
+        kernels.head_prepare_many(*calls)  # (convolution, norm, rotation, queries and the cache's keys and values: one launch)
+        if self.conv is not None:
+            self.conv.keep_inputs(ctx, u, state.state if state is not None else None)
         att = ctx.scratch((T, H2 * hd), ctx.dtype)
         kernels.attend(ctx, att, q, cache, H2, G2, hd, self.scale)
         width = self.n_heads * self.value_dim

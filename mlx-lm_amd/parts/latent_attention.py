@@ -108,12 +108,12 @@ class LatentAttention(Mixer):
         if writes_cache:
             if not self.own_latent:
                 raise RuntimeError("a latent-attention layer without a down-projection reads another layer's cache slot")
-            c = ctx.scratch((T, hd), ctx.dtype)
-            calls.append((c, u, Q + H, 1, r + dr, dict(dst_stride=hd, dst_fill=hd, norm_dim=r, norm_weight=self.c_norm,
-                                                       eps=self.eps, **rot)))
+            # the latent goes straight to its pages, as the one key head's key and as its value
+            for values in (False, True):
+                pages = kernels.PagesOut(cache.kv, values, cache.block_table, ctx.token_req, ctx.positions)
+                calls.append((pages, u, Q + H, 1, r + dr, dict(dst_stride=hd, dst_fill=hd, norm_dim=r, norm_weight=self.c_norm,
+                                                               eps=self.eps, **rot)))
         kernels.head_prepare_many(*calls)  # (queries and the latent in one launch)
-        if writes_cache:
-            kernels.kv_write(c, c, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
         att = ctx.scratch((T, H * hd), ctx.dtype)
         kernels.attend(ctx, att, q, cache, H, 1, hd, self.scale)
         kernels.head_gate(att, hd, H, u[:, Q:Q + H])
