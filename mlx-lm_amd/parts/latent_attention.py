@@ -99,7 +99,10 @@ class LatentAttention(Mixer):
         kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
         Qp = -(-Q // 8) * 8
         cq = ctx.scratch((T, Qp), ctx.dtype)
-        kernels.head_prepare(cq, u, 0, 1, Q, dst_stride=Qp, dst_fill=Qp, norm_dim=Q, norm_weight=self.q_norm, eps=self.eps)
+        if Qp == Q:
+            kernels.rmsnorm(cq, u, self.q_norm, self.eps)  # (a block a row; the rows' first Q columns)
+        else:
+            kernels.head_prepare(cq, u, 0, 1, Q, dst_stride=Qp, dst_fill=Qp, norm_dim=Q, norm_weight=self.q_norm, eps=self.eps)
         qf = ctx.scratch((T, H * (r + dr)), torch.float32)
         kernels.linear(qf, cq, self.q_w, splits=kernels.splits_alone(T))
         rot = dict(rot_off=r, rot_dims=dr, inv_freq=self.inv_freq, rot_mult=self.rot_mult, positions=ctx.positions)
