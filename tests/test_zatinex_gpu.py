@@ -168,6 +168,37 @@ def test_two_maps_joined_and_heads_gated(dtype):
     assert (x.double().cpu().view(T, H, hd) - want).abs().max() <= tol
 
 
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_the_convolution_on_the_way_into_the_heads(taps):
+    """``head_prepare`` with a convolution ahead: two requests in portions of 2, 1, 1, 6 and 3 tokens
+    (shorter than the taps, so old inputs stay in the state; single tokens, where the kernel moves
+    the state up itself), the first tokens of a request seeing zeros; then the heads' norm."""
+    from mlx_lm_amd.ops import kernels
+
+    H, d, n = 3, 10, 13
+    C = H * d + 4  # (channels beyond the heads: the state's rows are as wide as the projection)
+    g = torch.Generator().manual_seed(taps)
+    u = [torch.randn(n, C, generator=g) for _ in range(2)]
+    w = torch.randn(C, taps, generator=g)
+    nw = 1 + 0.3 * torch.randn(d, generator=g)
+    state = torch.zeros(3, 5 + (taps - 1) * C).cuda()
+    want = [plain.rms_norm(plain.causal_conv(x.double(), w.double())[:, : H * d].reshape(n, H, d), nw.double(), 1e-4) for x in u]
+    at, got = 0, [[], []]
+    for m in (2, 1, 1, 6, 3):
+        rows = torch.cat([u[0][at : at + m], u[1][at : at + m]]).cuda()
+        req, starts, slots = _ints([0] * m + [1] * m), _ints([0, m]), _ints([2, 1])
+        conv = kernels.ConvolutionAhead(w.cuda(), state, 5, req, starts, slots, single=m == 1)
+        out = torch.empty(2 * m, H * d, device="cuda")
+        kernels.head_prepare(out, rows, 0, H, d, norm_dim=d, norm_weight=nw.cuda(), eps=1e-4, conv=conv)
+        if m > 1:
+            kernels.conv_state_update(rows, 0, taps, C, state, 5, starts, _ints([m, m]), slots, 2)
+        got[0].append(out[:m].cpu()), got[1].append(out[m:].cpu())
+        at += m
+    for r in range(2):
+        assert (torch.cat(got[r]).double().view(n, H, d) - want[r]).abs().max() <= 2e-5
+    assert (state[0] == 0).all() and (state[:, :5] == 0).all()
+
+
 def _scan_channels(q, k, v, log_a, S):
     """``S = diag(a_t) S + k_t v_t^T; o_t = S^T q_t`` of one head, float64."""
     out = []
