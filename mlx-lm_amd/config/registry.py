@@ -7,7 +7,8 @@ MODEL_REMAPPING = {}
 
 _REGISTRY = {}
 _BUILTIN = {"gpt2": "mlx_lm_amd.models.gpt2", "pafutar": "mlx_lm_amd.models.pafutar",
-            "ruzolorn": "mlx_lm_amd.models.ruzolorn", "zatinex": "mlx_lm_amd.models.zatinex"}
+            "ruzolorn": "mlx_lm_amd.models.ruzolorn", "zatinex": "mlx_lm_amd.models.zatinex",
+            "sazilorn": "mlx_lm_amd.models.sazilorn"}
 
 
 def register_model(model_type, model_cls, args_cls):

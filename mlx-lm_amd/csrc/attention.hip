@@ -52,7 +52,20 @@ struct AttnArgs {
   const float* slopes;
   const void* gate;
   int ldg, keep_first;
+  //   softcap > 0: a scaled score s becomes softcap * tanh(s / softcap)
+  //   dist_bias [n_heads, n_dist]: dist_bias[h][min(query position - key position, n_dist - 1)] is added
+  float softcap;
+  const float* dist_bias;
+  int n_dist;
 };
+
+// A scaled score with the optional terms that depend on the head and the distance.
+__device__ __forceinline__ float shaped_score(const AttnArgs& p, float s, float slope, int h, int dist) {
+  if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
+  s -= slope * (float)dist;
+  if (p.dist_bias) s += p.dist_bias[(size_t)h * p.n_dist + min(max(dist, 0), p.n_dist - 1)];
+  return s;
+}
 
 // The two runs of keys that the queries at positions q_lo .. (whose last key is k_hi - 1) read:
 // the kept first keys [0, sink_hi) and the window's [k_lo, k_hi).  Without a window: one run.
@@ -275,7 +288,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnArgs p) {
         s += qv.x * krow[d] + qv.y * krow[d + 1] + qv.z * krow[d + 2] + qv.w * krow[d + 3];
       }
       const bool ok = qi < nq && kpos >= k_lo && kpos < k_hi && sees(p, qpos, kpos);
-      s = ok ? s - slope * (float)(qpos - kpos) : -INFINITY;
+      s = ok ? shaped_score(p, s, slope, h, qpos - kpos) : -INFINITY;
       const float m_new = fmaxf(m[i], wave_max(s));
       float pr = 0.f, alpha = 1.f;
       if (m_new != -INFINITY) {
@@ -531,7 +544,7 @@ __global__ __launch_bounds__(256) void attn_row_kernel(AttnArgs p) {
         s += qv.x * krow[d] + qv.y * krow[d + 1] + qv.z * krow[d + 2] + qv.w * krow[d + 3];
       }
       const bool ok = kpos >= k_lo && kpos < k_hi;
-      s = ok ? s - slope * (float)(pos - kpos) : -INFINITY;
+      s = ok ? shaped_score(p, s, slope, h, pos - kpos) : -INFINITY;
       const float m_new = fmaxf(m, wave_max(s));
       float pr = 0.f, alpha = 1.f;
       if (m_new != -INFINITY) {
@@ -691,6 +704,7 @@ static int fill_args(AttnArgs& p, const char* who, void* out, const void* q, int
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.head_dim = head_dim, p.page_size = page_size;
   p.window = window, p.n_splits = 1, p.scale = scale;
   p.head_scale = nullptr, p.slopes = nullptr, p.gate = nullptr, p.ldg = 0, p.keep_first = 0;
+  p.softcap = 0.f, p.dist_bias = nullptr, p.n_dist = 0;
   return 0;
 }
 
@@ -703,7 +717,17 @@ static int fill_extras(AttnArgs& p, const char* who, const float* head_scale, co
   p.keep_first = p.window > 0 ? keep_first : 0;  // (without a window every key is visible anyway)
   return 0;
 }
-static bool has_extras(const AttnArgs& p) { return p.head_scale || p.slopes || p.gate || p.keep_first > 0; }
+static bool has_extras(const AttnArgs& p) {
+  return p.head_scale || p.slopes || p.gate || p.keep_first > 0 || p.softcap > 0.f || p.dist_bias;
+}
+// The terms that only the `_terms` entry points bring.
+static int fill_shape(AttnArgs& p, const char* who, const AttnTerms* t) {
+  if (!t) return 0;
+  if (t->softcap < 0.f) FAIL("%s: softcap %g must not be negative", who, (double)t->softcap);
+  if (t->dist_bias && t->n_dist <= 0) FAIL("%s: a distance table of %d entries a head", who, t->n_dist);
+  p.softcap = t->softcap, p.dist_bias = t->dist_bias, p.n_dist = t->n_dist;
+  return 0;
+}
 
 // Kernels that want more than 64 KB of LDS have to be told so once per size.
 static int allow_lds(const char* who, const void* kernel, size_t bytes) {
@@ -726,13 +750,13 @@ static int allow_lds(const char* who, const void* kernel, size_t bytes) {
 // tile are consecutive tokens of one request at consecutive positions.
 // attn_tile_biased: attn_tile with the optional terms of AttnArgs (per-head scales, distance
 // slopes, kept first keys, an output gate; null or 0 where a term is absent).
-extern "C" int attn_tile_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                                const void* v_pages, size_t page_stride, const int* block_table,
-                                int max_blocks, const int* token_req, const int* positions,
-                                const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
-                                int page_size, int window, float scale, int dtype, const float* head_scale,
-                                const float* slopes, const void* gate, int ldg, int keep_first,
-                                hipStream_t stream) {
+static int tile_launch(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                       const void* v_pages, size_t page_stride, const int* block_table,
+                       int max_blocks, const int* token_req, const int* positions,
+                       const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
+                       int page_size, int window, float scale, int dtype, const float* head_scale,
+                       const float* slopes, const void* gate, int ldg, int keep_first, const AttnTerms* shape,
+                       hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   AttnArgs p;
   if (fill_args(p, "attn_tile", out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table,
@@ -740,6 +764,7 @@ extern "C" int attn_tile_biased(void* out, const void* q, int ldq, int ldo, cons
                 window, scale, dtype))
     return 1;
   if (fill_extras(p, "attn_tile", head_scale, slopes, gate, ldg, keep_first)) return 1;
+  if (fill_shape(p, "attn_tile", shape)) return 1;
   if (!has_extras(p) && dtype == DT_F32 && (head_dim == 64 || head_dim == 128) && page_size % 16 == 0 && ldq % 4 == 0 &&
       ldo % 4 == 0 && (((uintptr_t)q | (uintptr_t)out) & 15) == 0) {
     dim3 grid((n_tiles + 3) / 4, n_heads), block(256);
@@ -763,6 +788,31 @@ extern "C" int attn_tile_biased(void* out, const void* q, int ldq, int ldo, cons
   return 0;
 }
 
+extern "C" int attn_tile_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                const void* v_pages, size_t page_stride, const int* block_table,
+                                int max_blocks, const int* token_req, const int* positions,
+                                const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
+                                int page_size, int window, float scale, int dtype, const float* head_scale,
+                                const float* slopes, const void* gate, int ldg, int keep_first,
+                                hipStream_t stream) {
+  return tile_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req, positions,
+                     tiles, n_tiles, n_heads, n_kv_heads, head_dim, page_size, window, scale, dtype, head_scale,
+                     slopes, gate, ldg, keep_first, nullptr, stream);
+}
+
+// attn_tile_terms: every optional term, as an AttnTerms (attention_tiles.h); null: none.
+extern "C" int attn_tile_terms(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                               const void* v_pages, size_t page_stride, const int* block_table,
+                               int max_blocks, const int* token_req, const int* positions,
+                               const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
+                               int page_size, int window, float scale, int dtype, const AttnTerms* t,
+                               hipStream_t stream) {
+  return tile_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req, positions,
+                     tiles, n_tiles, n_heads, n_kv_heads, head_dim, page_size, window, scale, dtype,
+                     t ? t->head_scale : nullptr, t ? t->slopes : nullptr, t ? t->gate : nullptr, t ? t->ldg : 0,
+                     t ? t->keep_first : 0, t, stream);
+}
+
 extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                          const void* v_pages, size_t page_stride, const int* block_table,
                          int max_blocks, const int* token_req, const int* positions,
@@ -776,13 +826,13 @@ extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void*
 // rows: n_rows flat row indices, each handled as a single query.  With
 // n_splits > 1 the caller gives part_o [n_rows*n_heads*n_splits*head_dim] and
 // part_ml [n_rows*n_heads*n_splits*2] floats.
-extern "C" int attn_row_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                               const void* v_pages, size_t page_stride, const int* block_table,
-                               int max_blocks, const int* token_req, const int* positions,
-                               const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
-                               int page_size, int window, float scale, int n_splits, float* part_o,
-                               float* part_ml, int dtype, const float* head_scale, const float* slopes,
-                               const void* gate, int ldg, int keep_first, hipStream_t stream) {
+static int row_launch(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                      const void* v_pages, size_t page_stride, const int* block_table,
+                      int max_blocks, const int* token_req, const int* positions,
+                      const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                      int page_size, int window, float scale, int n_splits, float* part_o,
+                      float* part_ml, int dtype, const float* head_scale, const float* slopes,
+                      const void* gate, int ldg, int keep_first, const AttnTerms* shape, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   AttnArgs p;
   if (fill_args(p, "attn_row", out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table,
@@ -790,6 +840,7 @@ extern "C" int attn_row_biased(void* out, const void* q, int ldq, int ldo, const
                 window, scale, dtype))
     return 1;
   if (fill_extras(p, "attn_row", head_scale, slopes, gate, ldg, keep_first)) return 1;
+  if (fill_shape(p, "attn_row", shape)) return 1;
   if (n_splits < 1 || n_splits > 65535) FAIL("attn_row: n_splits %d out of range", n_splits);
   if (n_splits > 1 && (!part_o || !part_ml)) FAIL("attn_row: splits need the partial buffers");
   p.n_splits = n_splits, p.part_o = part_o, p.part_ml = part_ml;
@@ -809,6 +860,31 @@ extern "C" int attn_row_biased(void* out, const void* q, int ldq, int ldo, const
   }
   CHECK_LAUNCH("attn_row");
   return 0;
+}
+
+extern "C" int attn_row_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                               const void* v_pages, size_t page_stride, const int* block_table,
+                               int max_blocks, const int* token_req, const int* positions,
+                               const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                               int page_size, int window, float scale, int n_splits, float* part_o,
+                               float* part_ml, int dtype, const float* head_scale, const float* slopes,
+                               const void* gate, int ldg, int keep_first, hipStream_t stream) {
+  return row_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req, positions,
+                    rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale, n_splits, part_o, part_ml,
+                    dtype, head_scale, slopes, gate, ldg, keep_first, nullptr, stream);
+}
+
+// attn_row_terms: every optional term, as an AttnTerms (attention_tiles.h); null: none.
+extern "C" int attn_row_terms(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                              const void* v_pages, size_t page_stride, const int* block_table,
+                              int max_blocks, const int* token_req, const int* positions,
+                              const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                              int page_size, int window, float scale, int n_splits, float* part_o,
+                              float* part_ml, int dtype, const AttnTerms* t, hipStream_t stream) {
+  return row_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req, positions,
+                    rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale, n_splits, part_o, part_ml,
+                    dtype, t ? t->head_scale : nullptr, t ? t->slopes : nullptr, t ? t->gate : nullptr, t ? t->ldg : 0,
+                    t ? t->keep_first : 0, t, stream);
 }
 
 extern "C" int attn_row(void* out, const void* q, int ldq, int ldo, const void* k_pages,

@@ -22,6 +22,7 @@
 // columns of *its* keys and is only joined over the lane groups (and then the
 // waves) at the end.
 #include "common.h"
+#include "attention_tiles.h"
 
 struct DecodeArgs {
   void* out;  // out, q and the pages hold the kernel's element type
@@ -61,6 +62,11 @@ struct DecodeArgs {
   const float* slopes;
   const void* gate;
   int ldg, keep_first;
+  // softcap > 0: a scaled score s becomes softcap * tanh(s / softcap); dist_bias [n_heads, n_dist]:
+  // dist_bias[h][min(distance, n_dist - 1)] is added to a score
+  float softcap;
+  const float* dist_bias;
+  int n_dist;
 };
 
 template <typename T>
@@ -256,7 +262,10 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
       for (int i = 0; i < EPL; ++i) d += qf[i] * kf[i];
       d = group_sum<CPK>(d);  // over the key's lanes
       const int key = kt + j * KPL + kin;
-      s[j] = (key >= t_lo && key < t_hi) ? d - slope * (float)(pos - key) : -INFINITY;
+      if (p.softcap > 0.f) d = p.softcap * tanhf(d / p.softcap);
+      d -= slope * (float)(pos - key);
+      if (p.dist_bias) d += p.dist_bias[(size_t)h * p.n_dist + min(max(pos - key, 0), p.n_dist - 1)];
+      s[j] = (key >= t_lo && key < t_hi) ? d : -INFINITY;
       tmax = fmaxf(tmax, s[j]);
     }
     tmax = wave_max(tmax);
@@ -537,17 +546,18 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, h
 // 65,536 (row, head)s; part_o and part_ml are still where the parts pass through); 2, the same,
 // and n_splits is only the most a row takes: a short row takes fewer, by its own length.
 // Launches that join in the kernel and overlap on one GPU race (they share the counters).
-// attn_decode_rows_biased: with the optional terms of DecodeArgs (null or 0 where one is absent).
-extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                                       const void* v_pages, size_t page_stride, const int* block_table,
-                                       int max_blocks, const int* token_req, const int* positions,
-                                       const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
-                                       int page_size, int window, float scale, int n_splits, float* part_o,
-                                       float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
-                                       int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
-                                       int join_in_kernel, const float* head_scale, const float* slopes,
-                                       const void* gate, int ldg, int keep_first, hipStream_t stream) {
+static int decode_rows_launch(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                              const void* v_pages, size_t page_stride, const int* block_table,
+                              int max_blocks, const int* token_req, const int* positions,
+                              const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                              int page_size, int window, float scale, int n_splits, float* part_o,
+                              float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                              int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
+                              int join_in_kernel, const float* head_scale, const float* slopes,
+                              const void* gate, int ldg, int keep_first, const AttnTerms* shape, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (shape && (shape->softcap < 0.f || (shape->dist_bias && shape->n_dist <= 0)))
+    FAIL("attn_decode: softcap %g, a distance table of %d entries a head", (double)shape->softcap, shape->n_dist);
   if (keep_first < 0) FAIL("attn_decode: keep_first %d must not be negative", keep_first);
   if (gate && ldg < n_heads * head_dim) FAIL("attn_decode: the gate's row stride %d is smaller than its rows", ldg);
   if (key_tile == 0) key_tile = 32;
@@ -583,6 +593,8 @@ extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ld
   p.window = window, p.n_splits = n_splits, p.scale = scale;
   p.head_scale = head_scale, p.slopes = slopes, p.gate = gate, p.ldg = ldg;
   p.keep_first = window > 0 ? keep_first : 0;
+  p.softcap = shape ? shape->softcap : 0.f, p.dist_bias = shape ? shape->dist_bias : nullptr;
+  p.n_dist = shape ? shape->n_dist : 0;
   if (ahead && (((uintptr_t)ahead & 15) || ahead_chunk_bytes % 16 != 0 || ahead_chunks < 0))
     FAIL("attn_decode: what is read ahead must be chunks of 16-byte pieces");
   p.ahead = (const uint4*)ahead, p.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;
@@ -615,6 +627,40 @@ extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ld
   }
   CHECK_LAUNCH("attn_decode");
   return 0;
+}
+
+// attn_decode_rows_biased: with the optional terms of DecodeArgs (null or 0 where one is absent).
+extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                       const void* v_pages, size_t page_stride, const int* block_table,
+                                       int max_blocks, const int* token_req, const int* positions,
+                                       const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                                       int page_size, int window, float scale, int n_splits, float* part_o,
+                                       float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                                       int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
+                                       int join_in_kernel, const float* head_scale, const float* slopes,
+                                       const void* gate, int ldg, int keep_first, hipStream_t stream) {
+  return decode_rows_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                            positions, rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                            n_splits, part_o, part_ml, n_waves, ahead, ahead_chunk_bytes, ahead_chunks,
+                            rows_are_requests, dtype, key_tile, join_in_kernel, head_scale, slopes, gate, ldg,
+                            keep_first, nullptr, stream);
+}
+
+// attn_decode_rows_terms: every optional term, as an AttnTerms (attention_tiles.h); null: none.
+extern "C" int attn_decode_rows_terms(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                      const void* v_pages, size_t page_stride, const int* block_table,
+                                      int max_blocks, const int* token_req, const int* positions,
+                                      const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                                      int page_size, int window, float scale, int n_splits, float* part_o,
+                                      float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                                      int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
+                                      int join_in_kernel, const AttnTerms* t, hipStream_t stream) {
+  return decode_rows_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                            positions, rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                            n_splits, part_o, part_ml, n_waves, ahead, ahead_chunk_bytes, ahead_chunks,
+                            rows_are_requests, dtype, key_tile, join_in_kernel, t ? t->head_scale : nullptr,
+                            t ? t->slopes : nullptr, t ? t->gate : nullptr, t ? t->ldg : 0, t ? t->keep_first : 0, t,
+                            stream);
 }
 
 extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,

@@ -48,6 +48,11 @@ struct PrefillArgs {
   const float* slopes;
   const uint16_t* gate;
   int ldg, keep_first;
+  // softcap > 0: a scaled score s becomes softcap * tanh(s / softcap); dist_bias [n_heads, n_dist]:
+  // dist_bias[h][min(distance, n_dist - 1)] is added to a score (the kernel's SHAPED variant)
+  float softcap;
+  const float* dist_bias;
+  int n_dist;
 };
 
 #define BQ ATTN_PREFILL_TILE_QUERIES  // queries per block
@@ -67,7 +72,8 @@ __device__ __forceinline__ int key_of_row(int rho) {
 
 // POW2: the page size is a power of two (a key's page and row are a shift and a mask)
 // EXTRAS: the optional terms of PrefillArgs are looked at (the plain variant has no trace of them)
-template <int HD, bool POW2, bool EXTRAS>
+// SHAPED (with EXTRAS): scores also pass the soft cap and take the distance table's term
+template <int HD, bool POW2, bool EXTRAS, bool SHAPED = false>
 __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(PrefillArgs p) {
   constexpr int KS_STRIDE = HD + 8;
   constexpr int DC = HD / 16;           // 16-column chunks of a head (QK contraction steps)
@@ -260,7 +266,26 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
       const bool all_seen = sink ? kt + KT <= sink_hi
                                  : (kt >= k_lo && kt + KT - 1 <= wave_q0 && wave_q0 + 31 < nq + pos0 &&
                                     (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
-      if (all_seen) {
+      if constexpr (SHAPED) {
+        // the score in its own units first: the cap and the table's term are no linear function of it
+        const int run_lo = sink ? 0 : k_lo, run_hi = sink ? sink_hi : k_hi;
+        const float c1 = p.head_scale ? p.head_scale[h] : p.scale;
+        const float* bias_row = p.dist_bias ? p.dist_bias + (size_t)h * p.n_dist : nullptr;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int o = 32 * s + 16 * (r >> 3) + (r & 7);
+            const int key = kt + 8 * g + o;
+            const bool ok = q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first);
+            float v = st[s][r] * c1;
+            if (p.softcap > 0.f) v = p.softcap * tanhf(v / p.softcap);
+            if (bias_row) v += bias_row[min(max(qpos - key, 0), p.n_dist - 1)];
+            v = fmaf(v, 1.4426950408889634f, fmaf(slope2, (float)o, -far));
+            st[s][r] = ok ? v : -INFINITY;
+            tmax = fmaxf(tmax, st[s][r]);
+          }
+      } else if (all_seen) {
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -406,15 +431,16 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 // tiles: n_tiles pairs (first flat row, number of rows 1..128); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
 // bfloat16 only, head_dim 32, 64, 128 or 256.
-// attn_prefill_biased: with the optional terms of PrefillArgs (null or 0 where one is absent).
-extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                                   const void* v_pages, size_t page_stride, const int* block_table,
-                                   int max_blocks, const int* token_req, const int* positions,
-                                   const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
-                                   int head_dim, int page_size, int window, float scale,
-                                   const float* head_scale, const float* slopes, const void* gate, int ldg,
-                                   int keep_first, hipStream_t stream) {
+static int prefill_launch(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                          const void* v_pages, size_t page_stride, const int* block_table,
+                          int max_blocks, const int* token_req, const int* positions,
+                          const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
+                          int head_dim, int page_size, int window, float scale,
+                          const float* head_scale, const float* slopes, const void* gate, int ldg,
+                          int keep_first, const AttnTerms* shape, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (shape && (shape->softcap < 0.f || (shape->dist_bias && shape->n_dist <= 0)))
+    FAIL("attn_prefill: softcap %g, a distance table of %d entries a head", (double)shape->softcap, shape->n_dist);
   if (keep_first < 0) FAIL("attn_prefill: keep_first %d must not be negative", keep_first);
   if (gate && (ldg < n_heads * head_dim || ldg % 4 != 0 || ((uintptr_t)gate & 7)))
     FAIL("attn_prefill: the gate's rows (stride %d) must be 8-byte aligned and as wide as the output's", ldg);
@@ -443,7 +469,10 @@ extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, c
   p.scale = scale;
   p.head_scale = head_scale, p.slopes = slopes, p.gate = (const uint16_t*)gate, p.ldg = ldg;
   p.keep_first = window > 0 ? keep_first : 0;
-  const bool extras = head_scale || slopes || gate || p.keep_first > 0;
+  p.softcap = shape ? shape->softcap : 0.f, p.dist_bias = shape ? shape->dist_bias : nullptr;
+  p.n_dist = shape ? shape->n_dist : 0;
+  const bool shaped = p.softcap > 0.f || p.dist_bias;
+  const bool extras = head_scale || slopes || gate || p.keep_first > 0 || shaped;
   if (n_tiles > 65535) FAIL("attn_prefill: %d tiles in a launch, at most 65535", n_tiles);
   dim3 grid(n_heads, n_tiles), block(256);
   // a request's page numbers lie in LDS beside the tiles
@@ -453,7 +482,10 @@ extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, c
   const size_t lds = (size_t)(max_blocks + (extras ? 2 : 0)) * sizeof(int);
   const bool pow2 = p.page_shift >= 0;
 #define LAUNCH_PREFILL(HD)                                                                                  \
-  if (extras) {                                                                                             \
+  if (shaped) {                                                                                             \
+    if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true, true, true>), grid, block, lds, stream, p); \
+    else hipLaunchKernelGGL((attn_prefill_kernel<HD, false, true, true>), grid, block, lds, stream, p);     \
+  } else if (extras) {                                                                                             \
     if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true, true>), grid, block, lds, stream, p);      \
     else hipLaunchKernelGGL((attn_prefill_kernel<HD, false, true>), grid, block, lds, stream, p);          \
   } else if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true, false>), grid, block, lds, stream, p); \
@@ -470,6 +502,32 @@ extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, c
 #undef LAUNCH_PREFILL
   CHECK_LAUNCH("attn_prefill");
   return 0;
+}
+
+// attn_prefill_biased: with the optional terms of PrefillArgs (null or 0 where one is absent).
+extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                   const void* v_pages, size_t page_stride, const int* block_table,
+                                   int max_blocks, const int* token_req, const int* positions,
+                                   const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
+                                   int head_dim, int page_size, int window, float scale,
+                                   const float* head_scale, const float* slopes, const void* gate, int ldg,
+                                   int keep_first, hipStream_t stream) {
+  return prefill_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req, positions,
+                        tiles, n_tiles, n_heads, n_kv_heads, head_dim, page_size, window, scale, head_scale, slopes,
+                        gate, ldg, keep_first, nullptr, stream);
+}
+
+// attn_prefill_terms: every optional term, as an AttnTerms (attention_tiles.h); null: none.
+extern "C" int attn_prefill_terms(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                  const void* v_pages, size_t page_stride, const int* block_table,
+                                  int max_blocks, const int* token_req, const int* positions,
+                                  const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
+                                  int head_dim, int page_size, int window, float scale, const AttnTerms* t,
+                                  hipStream_t stream) {
+  return prefill_launch(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req, positions,
+                        tiles, n_tiles, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                        t ? t->head_scale : nullptr, t ? t->slopes : nullptr, t ? t->gate : nullptr, t ? t->ldg : 0,
+                        t ? t->keep_first : 0, t, stream);
 }
 
 extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const void* k_pages,

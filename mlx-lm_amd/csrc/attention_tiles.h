@@ -2,6 +2,24 @@
 // sizes are written.  The kernels include it; who makes the lists asks eng_attn_tile_sizes().
 #pragma once
 
+// The optional terms of a score and of the output that the attention kernels' `_terms` entry
+// points take (a null pointer or 0 where a term is absent).  A score is made in this order:
+//   s = (q . k) * scale            (head_scale[h] instead of scale where given)
+//   s = softcap * tanh(s / softcap)                       (softcap > 0)
+//   s -= slopes[h] * (query position - key position)
+//   s += dist_bias[h * n_dist + min(distance, n_dist - 1)]      (a table of float, a row a head)
+// keep_first: with a window, the first so many keys stay visible.  gate (rows of stride ldg, the
+// queries' element type): the output is multiplied by its sigmoid.
+struct AttnTerms {
+  const float* head_scale;
+  const float* slopes;
+  const void* gate;
+  int ldg, keep_first;
+  float softcap;
+  const float* dist_bias;
+  int n_dist;
+};
+
 #define ATTN_TILE_QUERIES 16           // attn_tile (attention.hip): queries a block
 #define ATTN_PREFILL_TILE_QUERIES 128  // attn_prefill (attention_prefill.hip): queries a block
 

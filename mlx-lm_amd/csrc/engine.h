@@ -187,6 +187,10 @@ int eng_ffn_forward(EngPart* ffn, EngCtx* ctx, const EngValue* x, const EngMat* 
 // attention of the step's queries over a slot's pages, the kernels chosen as the attention part does
 int eng_attend(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads, int head_dim,
                int window, float scale, int array_base);
+// the same with the optional terms of a score and of the output (struct AttnTerms, attention_tiles.h)
+struct AttnTerms;
+int eng_attend_terms(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads,
+                     int head_dim, int window, float scale, int array_base, const struct AttnTerms* terms);
 int eng_embedding_forward(EngPart* embedding, EngCtx* ctx, const EngMat* out, EngPart* positions);
 int eng_head_forward(EngPart* head, EngCtx* ctx, const EngValue* x, const EngMat* out);
 int eng_settle(EngCtx* ctx);

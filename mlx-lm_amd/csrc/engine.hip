@@ -118,6 +118,21 @@ typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const 
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
 
+// (the same with the optional score terms: an AttnTerms ahead of the stream)
+typedef int (*fn_attn_tile_terms)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
+                                  const int*, const int*, const int*, int, int, int, int, int, int, float, int,
+                                  const AttnTerms*, hipStream_t);
+typedef int (*fn_attn_row_terms)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
+                                 const int*, const int*, const int*, int, int, int, int, int, int, float, int,
+                                 float*, float*, int, const AttnTerms*, hipStream_t);
+typedef int (*fn_attn_decode_terms)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
+                                    const int*, const int*, const int*, int, int, int, int, int, int, float, int,
+                                    float*, float*, int, const void*, size_t, int, int, int, int, int,
+                                    const AttnTerms*, hipStream_t);
+typedef int (*fn_attn_prefill_terms)(void*, const void*, int, int, const void*, const void*, size_t, const int*,
+                                     int, const int*, const int*, const int*, int, int, int, int, int, int, float,
+                                     const AttnTerms*, hipStream_t);
+
 static Entry<fn_embed> k_embed("embed", "embed_scale_add");
 static Entry<fn_layernorm> k_layernorm("norm", "layernorm");
 static Entry<int (*)(void*, const float*, int, const int*, const float*, float, int, int, int, hipStream_t)> k_rmsnorm("rmsnorm", "rmsnorm");
@@ -141,6 +156,10 @@ static Entry<fn_attn_row> k_attn_row("attention", "attn_row");
 static Entry<fn_attn_decode> k_attn_decode("attention_decode", "attn_decode_rows");
 static Entry<fn_attn_decode_group> k_attn_decode_group("attention_decode", "attn_decode_group");
 static Entry<fn_attn_prefill> k_attn_prefill("attention_prefill", "attn_prefill");
+static Entry<fn_attn_tile_terms> k_attn_tile_terms("attention", "attn_tile_terms");
+static Entry<fn_attn_row_terms> k_attn_row_terms("attention", "attn_row_terms");
+static Entry<fn_attn_decode_terms> k_attn_decode_terms("attention_decode", "attn_decode_rows_terms");
+static Entry<fn_attn_prefill_terms> k_attn_prefill_terms("attention_prefill", "attn_prefill_terms");
 
 // Launch through an entry: a missing library or a refused call becomes this library's error.
 #define KERNEL(entry, ctx, ...)                                                                  \
@@ -754,7 +773,11 @@ struct Attention : Mixer {
            (key_bytes == 64 || key_bytes == 128 || key_bytes == 256) && kv.page_size % (1024 / key_bytes) == 0;
   }
 
-  int attend(EngCtx* ctx, const EngMat& out, const EngMat& q, const EngScatter& kv, bool out_packed) const {
+  // `terms`: the optional terms of a score and of the output (attention_tiles.h), or null.  With
+  // terms the kernels' `_terms` entry points are called; the kernel that takes the query heads of
+  // a key head together knows no terms, so such rows go to the streaming kernel.
+  int attend(EngCtx* ctx, const EngMat& out, const EngMat& q, const EngScatter& kv, bool out_packed,
+             const AttnTerms* terms = nullptr) const {
     const int* tiles = ctx->arrays[array_base + ARR_TILES];
     const int* rows = ctx->arrays[array_base + ARR_ROWS];
     const int* all_tiles = ctx->arrays[array_base + ARR_ALL_TILES];
@@ -772,13 +795,27 @@ struct Attention : Mixer {
     // than the row kernel takes go to the general tile kernel, rows and all)
     const bool wide_fast = bf16 && head_dim == 256 && kv.page_size % 2 == 0;
     if (head_dim > ATTN_ROW_MAX_HEAD_DIM && !wide_fast) {
-      KERNEL(k_attn_tile, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks,
-             kv.token_req, kv.positions, all_tiles, n_all_tiles, n_heads, n_kv_heads, head_dim, kv.page_size,
-             window, scale, q.dtype, ctx->stream);
+      if (terms)
+        KERNEL(k_attn_tile_terms, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
+               kv.max_blocks, kv.token_req, kv.positions, all_tiles, n_all_tiles, n_heads, n_kv_heads, head_dim,
+               kv.page_size, window, scale, q.dtype, terms, ctx->stream);
+      else
+        KERNEL(k_attn_tile, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks,
+               kv.token_req, kv.positions, all_tiles, n_all_tiles, n_heads, n_kv_heads, head_dim, kv.page_size,
+               window, scale, q.dtype, ctx->stream);
       return 0;
     }
     const bool mfma_sizes = bf16 && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
-    if (n_tiles) {
+    if (n_tiles && terms) {
+      if (mfma_sizes)
+        KERNEL(k_attn_prefill_terms, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
+               kv.max_blocks, kv.token_req, kv.positions, big_tiles, n_big_tiles, n_heads, n_kv_heads, head_dim,
+               kv.page_size, window, scale, terms, ctx->stream);
+      else
+        KERNEL(k_attn_tile_terms, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
+               kv.max_blocks, kv.token_req, kv.positions, tiles, n_tiles, n_heads, n_kv_heads, head_dim,
+               kv.page_size, window, scale, q.dtype, terms, ctx->stream);
+    } else if (n_tiles) {
       if (mfma_sizes)
         KERNEL(k_attn_prefill, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, big_tiles, n_big_tiles, n_heads, n_kv_heads, head_dim,
@@ -799,7 +836,7 @@ struct Attention : Mixer {
       // A block is four waves of sixteen keys at a time; a part for every 128 keys of the longest
       // row, as many as give every CU two blocks.
       const int group = n_heads / n_kv_heads;
-      if (bf16 && group >= 8 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
+      if (!terms && bf16 && group >= 8 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
         const long c = window <= 0 ? max_row_context : (max_row_context < window + 15 ? max_row_context : window + 15);
         const long blocks = (long)n_rows * n_kv_heads * ((group + 15) / 16);
         long ns = c / 128, most = 2L * ctx->n_compute_units / (blocks < 1 ? 1 : blocks);
@@ -845,11 +882,23 @@ struct Attention : Mixer {
         } else {
           ahead = nullptr;
         }
-        KERNEL(k_attn_decode, ctx, out.p, q.p, q.ld, out_packed ? 0 : out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
+        if (terms)
+          KERNEL(k_attn_decode_terms, ctx, out.p, q.p, q.ld, out_packed ? 0 : out.ld, kv.k, kv.v, kv.page_stride,
+                 kv.block_table, kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
+                 kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
+                 ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
+                 q.dtype, key_tile, 2, terms, ctx->stream);
+        else
+          KERNEL(k_attn_decode, ctx, out.p, q.p, q.ld, out_packed ? 0 : out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
+                 kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
+                 kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
+                 ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
+                 q.dtype, key_tile, 2, ctx->stream);
+      } else if (terms) {
+        KERNEL(k_attn_row_terms, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
-               kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
-               ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
-               q.dtype, key_tile, 2, ctx->stream);
+               kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, q.dtype, terms,
+               ctx->stream);
       } else {
         KERNEL(k_attn_row, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
@@ -1236,8 +1285,8 @@ extern "C" int eng_mixer_forward(EngPart* mixer, EngCtx* ctx, const EngValue* x,
 // among the attention kernels that the built-in attention part makes (rows to the decode kernels,
 // portions to the tile kernels, by the step's work lists from `array_base` on): for a mixer that
 // prepares queries, keys and values in its own way and wants only this.
-extern "C" int eng_attend(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads,
-                          int head_dim, int window, float scale, int array_base) {
+static int attend_slot(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads,
+                       int head_dim, int window, float scale, int array_base, const AttnTerms* terms) {
   if (!out || !q || n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads)
     FAIL("eng_attend: %d query heads over %d key heads", n_heads, n_kv_heads);
   if (array_base < 0 || array_base + ARR_ROWS_ARE_REQUESTS >= ENG_MAX_ARRAYS)
@@ -1250,7 +1299,19 @@ extern "C" int eng_attend(EngCtx* ctx, const EngMat* out, const EngMat* q, int s
   a.qkv_w = EngWeight{}, a.out_w = EngWeight{}, a.qkv_b = a.out_b = nullptr, a.position = nullptr;
   EngScatter kv;
   TRY(a.scatter_for(ctx, slot, &kv));
-  return a.attend(ctx, *out, *q, kv, false);
+  if (terms && terms->gate && terms->ldg < q->cols) FAIL("eng_attend: the gate's rows are shorter than the queries'");
+  return a.attend(ctx, *out, *q, kv, false, terms);
+}
+
+extern "C" int eng_attend(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads,
+                          int head_dim, int window, float scale, int array_base) {
+  return attend_slot(ctx, out, q, slot, n_heads, n_kv_heads, head_dim, window, scale, array_base, nullptr);
+}
+
+// eng_attend with the optional terms of a score and of the output (AttnTerms, attention_tiles.h).
+extern "C" int eng_attend_terms(EngCtx* ctx, const EngMat* out, const EngMat* q, int slot, int n_heads, int n_kv_heads,
+                                int head_dim, int window, float scale, int array_base, const AttnTerms* terms) {
+  return attend_slot(ctx, out, q, slot, n_heads, n_kv_heads, head_dim, window, scale, array_base, terms);
 }
 
 extern "C" int eng_ffn_forward(EngPart* ffn, EngCtx* ctx, const EngValue* x, const EngMat* residual) {

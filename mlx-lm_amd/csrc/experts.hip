@@ -25,8 +25,10 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 // A wave a token, up to ROUTER_PER_LANE outputs a lane.  The k-th pick is the largest choice score
 // not picked yet, the lowest index on a tie.
 #define ROUTER_PER_LANE 8
+// `renorm`: the picks' weights are divided by their sum (+ 1e-20); `mult`: and multiplied by this.
 __device__ __forceinline__ void route_token(const float* __restrict__ zr, const float* __restrict__ correction, int n_out,
-                                            int top, int* __restrict__ idx, float* __restrict__ weight, int lane) {
+                                            int top, int* __restrict__ idx, float* __restrict__ weight, int lane,
+                                            int renorm = 0, float mult = 1.f) {
   float v[ROUTER_PER_LANE], c[ROUTER_PER_LANE];
   float m = -INFINITY;
 #pragma unroll
@@ -49,6 +51,10 @@ __device__ __forceinline__ void route_token(const float* __restrict__ zr, const 
     v[i] *= inv;
     c[i] = e < n_out ? (correction ? v[i] + correction[e] : v[i]) : -INFINITY;
   }
+  float mine[ROUTER_PER_LANE];  // pick j's weight, kept by lane j % 64 until the picks' sum is known
+#pragma unroll
+  for (int i = 0; i < ROUTER_PER_LANE; ++i) mine[i] = 0.f;
+  float total = 0.f;
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
 #pragma unroll
@@ -59,22 +65,32 @@ __device__ __forceinline__ void route_token(const float* __restrict__ zr, const 
     for (int i = ROUTER_PER_LANE - 1; i >= 0; --i)
       if (c[i] == best) first = -(float)(lane + 64 * i);
     const int e = (int)(-wave_max(first));
+    float w = 0.f;
 #pragma unroll
     for (int i = 0; i < ROUTER_PER_LANE; ++i)
       if (lane + 64 * i == e) {
-        idx[j] = e, weight[j] = v[i];
+        idx[j] = e, w = v[i];
         c[i] = -INFINITY;  // picked
       }
+    w = wave_sum(w);  // (one lane holds it)
+    total += w;
+#pragma unroll
+    for (int i = 0; i < ROUTER_PER_LANE; ++i)
+      if (lane == (j & 63) && i == (j >> 6)) mine[i] = w;
   }
+  const float factor = renorm ? mult / (total + 1e-20f) : mult;
+#pragma unroll
+  for (int i = 0; i < ROUTER_PER_LANE; ++i)
+    if (lane + 64 * i < top) weight[lane + 64 * i] = mine[i] * factor;
 }
 
 __global__ __launch_bounds__(256) void router_choice_kernel(const float* __restrict__ z, int ldz,
                                                             const float* __restrict__ correction, int n_tokens,
                                                             int n_out, int top, int* __restrict__ idx,
-                                                            float* __restrict__ weight) {
+                                                            float* __restrict__ weight, int renorm, float mult) {
   const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= n_tokens) return;  // whole waves leave; no barrier follows
-  route_token(z + (size_t)t * ldz, correction, n_out, top, idx + (size_t)t * top, weight + (size_t)t * top, lane);
+  route_token(z + (size_t)t * ldz, correction, n_out, top, idx + (size_t)t * top, weight + (size_t)t * top, lane, renorm, mult);
 }
 
 // For a step of few tokens, where one product gave [router | gate | up] as float rows: a block a
@@ -83,20 +99,23 @@ template <typename T>
 __global__ __launch_bounds__(256) void route_and_gate_kernel(const float* __restrict__ zu, int ld,
                                                              const float* __restrict__ correction, int n_out, int top,
                                                              int F, int* __restrict__ idx, float* __restrict__ weight,
-                                                             T* __restrict__ act, int ldo) {
+                                                             T* __restrict__ act, int ldo, int renorm, float mult) {
   const int t = blockIdx.x, lane = threadIdx.x & 63;
   const float* row = zu + (size_t)t * ld;
-  if (threadIdx.x < 64) route_token(row, correction, n_out, top, idx + (size_t)t * top, weight + (size_t)t * top, lane);
+  if (threadIdx.x < 64)
+    route_token(row, correction, n_out, top, idx + (size_t)t * top, weight + (size_t)t * top, lane, renorm, mult);
   for (int f = threadIdx.x; f < F; f += 256) act[(size_t)t * ldo + f] = from_f32<T>(silu_f(row[n_out + f]) * row[n_out + F + f]);
 }
 
-template <typename T>
+// GELU: the gate passes the tanh form of gelu instead of silu
+template <typename T, bool GELU>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gu, int ld, T* __restrict__ out, int ldo,
                                                        int n_rows, int F) {
   const int f = blockIdx.y * 256 + threadIdx.x, r = blockIdx.x;
   if (f >= F) return;
   const T* row = gu + (size_t)r * ld;
-  out[(size_t)r * ldo + f] = from_f32<T>(silu_f(to_f32(row[f])) * to_f32(row[F + f]));
+  const float z = to_f32(row[f]);
+  out[(size_t)r * ldo + f] = from_f32<T>((GELU ? gelu_tanh(z) : silu_f(z)) * to_f32(row[F + f]));
 }
 
 // ROWS dot products of one vector b with ROWS rows a[r] over a lane's share of K, all loads of a step on
@@ -444,20 +463,32 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(const float* __rest
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
-extern "C" int router_choice(const float* z, int ldz, const float* correction, int n_tokens, int n_out, int top,
-                             int* idx, float* weight, hipStream_t stream) {
+static int router_choice_launch(const float* z, int ldz, const float* correction, int n_tokens, int n_out, int top,
+                                int* idx, float* weight, int renorm, float mult, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (!z || !idx || !weight) FAIL("router_choice: null pointer");
   if (n_out <= 0 || top <= 0 || top > n_out || ldz < n_out) FAIL("router_choice: %d of %d outputs, rows of %d", top, n_out, ldz);
   if (n_out > 64 * ROUTER_PER_LANE) FAIL("router_choice: %d outputs, at most %d", n_out, 64 * ROUTER_PER_LANE);
   hipLaunchKernelGGL(router_choice_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, z, ldz, correction,
-                     n_tokens, n_out, top, idx, weight);
+                     n_tokens, n_out, top, idx, weight, renorm, mult);
   CHECK_LAUNCH("router_choice");
   return 0;
 }
 
-extern "C" int route_and_gate(const float* zu, int ld, const float* correction, int n_tokens, int n_out, int top, int F,
-                              int* idx, float* weight, void* act, int ldo, int dtype, hipStream_t stream) {
+extern "C" int router_choice(const float* z, int ldz, const float* correction, int n_tokens, int n_out, int top,
+                             int* idx, float* weight, hipStream_t stream) {
+  return router_choice_launch(z, ldz, correction, n_tokens, n_out, top, idx, weight, 0, 1.f, stream);
+}
+
+// router_choice_scaled: the picks' weights divided by their sum (+ 1e-20) where `renorm`, then times `mult`.
+extern "C" int router_choice_scaled(const float* z, int ldz, const float* correction, int n_tokens, int n_out, int top,
+                                    int* idx, float* weight, int renorm, float mult, hipStream_t stream) {
+  return router_choice_launch(z, ldz, correction, n_tokens, n_out, top, idx, weight, renorm, mult, stream);
+}
+
+static int route_and_gate_launch(const float* zu, int ld, const float* correction, int n_tokens, int n_out, int top, int F,
+                                 int* idx, float* weight, void* act, int ldo, int dtype, int renorm, float mult,
+                                 hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (!zu || !idx || !weight || !act) FAIL("route_and_gate: null pointer");
   if (n_out <= 0 || top <= 0 || top > n_out || F <= 0 || ld < n_out + 2 * F || ldo < F)
@@ -466,26 +497,56 @@ extern "C" int route_and_gate(const float* zu, int ld, const float* correction, 
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("route_and_gate: unknown dtype code %d", dtype);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(route_and_gate_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, zu, ld, correction, n_out, top, F,
-                       idx, weight, (float*)act, ldo);
+                       idx, weight, (float*)act, ldo, renorm, mult);
   else
     hipLaunchKernelGGL(route_and_gate_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, zu, ld, correction, n_out, top, F,
-                       idx, weight, (bf16*)act, ldo);
+                       idx, weight, (bf16*)act, ldo, renorm, mult);
   CHECK_LAUNCH("route_and_gate");
   return 0;
 }
 
-extern "C" int silu_mul(const void* gu, int ld, void* out, int ldo, int n_rows, int F, int dtype, hipStream_t stream) {
+extern "C" int route_and_gate(const float* zu, int ld, const float* correction, int n_tokens, int n_out, int top, int F,
+                              int* idx, float* weight, void* act, int ldo, int dtype, hipStream_t stream) {
+  return route_and_gate_launch(zu, ld, correction, n_tokens, n_out, top, F, idx, weight, act, ldo, dtype, 0, 1.f, stream);
+}
+
+extern "C" int route_and_gate_scaled(const float* zu, int ld, const float* correction, int n_tokens, int n_out, int top,
+                                     int F, int* idx, float* weight, void* act, int ldo, int dtype, int renorm, float mult,
+                                     hipStream_t stream) {
+  return route_and_gate_launch(zu, ld, correction, n_tokens, n_out, top, F, idx, weight, act, ldo, dtype, renorm, mult, stream);
+}
+
+// act_mul: out = act(gate) * up for rows [gate | up]; `activation` 0: silu, 1: the tanh form of gelu.
+static int act_mul_launch(const void* gu, int ld, void* out, int ldo, int n_rows, int F, int dtype, int activation,
+                          hipStream_t stream) {
   if (n_rows <= 0 || F <= 0) return 0;
+  if (activation != 0 && activation != 1) FAIL("act_mul: unknown activation code %d", activation);
   if (!gu || !out) FAIL("silu_mul: null pointer");
   if (ld < 2 * F || ldo < F) FAIL("silu_mul: rows of %d for 2 x %d, output rows of %d", ld, F, ldo);
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("silu_mul: unknown dtype code %d", dtype);
   dim3 grid(n_rows, (F + 255) / 256), block(256);
-  if (dtype == DT_F32)
-    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, ld, (float*)out, ldo, n_rows, F);
-  else
-    hipLaunchKernelGGL(silu_mul_kernel<bf16>, grid, block, 0, stream, (const bf16*)gu, ld, (bf16*)out, ldo, n_rows, F);
+  if (dtype == DT_F32) {
+    if (activation)
+      hipLaunchKernelGGL((silu_mul_kernel<float, true>), grid, block, 0, stream, (const float*)gu, ld, (float*)out, ldo, n_rows, F);
+    else
+      hipLaunchKernelGGL((silu_mul_kernel<float, false>), grid, block, 0, stream, (const float*)gu, ld, (float*)out, ldo, n_rows, F);
+  } else {
+    if (activation)
+      hipLaunchKernelGGL((silu_mul_kernel<bf16, true>), grid, block, 0, stream, (const bf16*)gu, ld, (bf16*)out, ldo, n_rows, F);
+    else
+      hipLaunchKernelGGL((silu_mul_kernel<bf16, false>), grid, block, 0, stream, (const bf16*)gu, ld, (bf16*)out, ldo, n_rows, F);
+  }
   CHECK_LAUNCH("silu_mul");
   return 0;
+}
+
+extern "C" int silu_mul(const void* gu, int ld, void* out, int ldo, int n_rows, int F, int dtype, hipStream_t stream) {
+  return act_mul_launch(gu, ld, out, ldo, n_rows, F, dtype, 0, stream);
+}
+
+extern "C" int act_mul(const void* gu, int ld, void* out, int ldo, int n_rows, int F, int dtype, int activation,
+                       hipStream_t stream) {
+  return act_mul_launch(gu, ld, out, ldo, n_rows, F, dtype, activation, stream);
 }
 
 // act: [n_tokens * top, F] of the compute dtype; y: float rows.

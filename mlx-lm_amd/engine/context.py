@@ -103,13 +103,14 @@ class CacheView:
     """One cache slot as a mixer sees it in a step: ``keys``/``values`` are the slot's pages
     (``[n_pages, n_kv_heads, page, width]`` each, of widths of their own), ``kv`` the same for the
     attention kernels here where both have one width, ``block_table`` the requests' page numbers,
-    ``state`` a slot of fixed-size state."""
+    ``state`` a slot of fixed-size state, of which this view's share starts ``offset`` floats into
+    a request's row (an arrangement that keeps state of its own ahead of its mixer's says so)."""
 
-    __slots__ = ("kv", "keys", "values", "block_table", "state", "slot")
+    __slots__ = ("kv", "keys", "values", "block_table", "state", "slot", "offset")
 
-    def __init__(self, slot, kv=None, block_table=None, state=None, keys=None, values=None):
+    def __init__(self, slot, kv=None, block_table=None, state=None, keys=None, values=None, offset=0):
         self.slot, self.kv, self.block_table, self.state = slot, kv, block_table, state
-        self.keys, self.values = keys, values
+        self.keys, self.values, self.offset = keys, values, int(offset)
 
 
 class HostBatch:
@@ -168,6 +169,7 @@ class StepContext:
         self.q_starts, self.q_lens, self.context_lens, self.state_slots = [], [], [], []
         self._views = {}
         self._kept = []  # tensors that the native side holds pointers to until the step is over
+        self.shared = {}  # what a layer leaves for later layers of the same step (scratch memory it did not give back)
         self._meta = None  # the device buffer that holds the step's integer arrays
         # a projection's sum into the residual stream that the next norm will add
         self.pending = PendingSum(self.c.pending, self)

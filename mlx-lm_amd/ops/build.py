@@ -23,7 +23,7 @@ CSRC = os.path.join(_PKG, "csrc")
 
 SOURCES = ("embed", "norm", "rmsnorm", "gemm_f32", "gemm_bf16", "gemm_bf16_decode", "attention", "attention_decode",
            "attention_prefill", "gated_key_attention", "relu2_mlp", "post_norm_block", "sandwich_block", "head_norm",
-           "linear_state", "head_prepare", "experts", "sampling", "engine")
+           "linear_state", "head_prepare", "experts", "parallel_block", "state_gates", "sampling", "engine")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

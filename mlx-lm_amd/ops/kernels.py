@@ -586,15 +586,40 @@ def kv_write(k_src, v_src, kv, block_table, token_req, positions):
     build.check(lib, rc, "kv_write")
 
 
+class AttnTerms(ctypes.Structure):
+    """Mirror of ``AttnTerms`` in csrc/attention_tiles.h."""
+
+    _fields_ = [("head_scale", _vp), ("slopes", _vp), ("gate", _vp), ("ldg", _c_int), ("keep_first", _c_int),
+                ("softcap", _c_float), ("dist_bias", _vp), ("n_dist", _c_int)]
+
+
 class ScoreTerms:
     """Optional terms that the four attention kernels take beside the plain causal scores:
     ``head_scale`` (float32 ``[n_heads]``, instead of ``scale``), ``slopes`` (float32 ``[n_heads]``:
     ``slope * (query position - key position)`` is taken off a score), ``gate`` (``[tokens,
-    n_heads * head_dim]`` of the queries' dtype: the output is multiplied by its sigmoid) and
-    ``keep_first`` (with a window, the first so many keys stay visible)."""
+    n_heads * head_dim]`` of the queries' dtype: the output is multiplied by its sigmoid),
+    ``keep_first`` (with a window, the first so many keys stay visible), ``softcap`` (a scaled
+    score ``s`` becomes ``softcap * tanh(s / softcap)``) and ``distance_bias`` (float32 ``[n_heads,
+    n]``: entry ``min(distance, n - 1)`` of the head's row is added to a score).  A score takes
+    them in this order: scale, cap, slope, table."""
 
-    def __init__(self, head_scale=None, slopes=None, gate=None, keep_first=0):
+    def __init__(self, head_scale=None, slopes=None, gate=None, keep_first=0, softcap=0.0, distance_bias=None):
         self.head_scale, self.slopes, self.gate, self.keep_first = head_scale, slopes, gate, int(keep_first)
+        self.softcap, self.distance_bias = float(softcap), distance_bias
+
+    def struct(self, q, n_heads):
+        """The terms as the kernels' ``_terms`` entry points and the native host take them."""
+        a = self.args(q, n_heads)
+        t = AttnTerms()
+        t.head_scale, t.slopes, t.gate = _ptr(self.head_scale), _ptr(self.slopes), _ptr(self.gate)
+        t.ldg, t.keep_first, t.softcap = a[3].value, self.keep_first, self.softcap
+        _need(self.softcap >= 0.0, "softcap must not be negative")
+        if self.distance_bias is not None:
+            _dev(self.distance_bias, "distance_bias", torch.float32)
+            _need(self.distance_bias.dim() == 2 and self.distance_bias.shape[0] == n_heads and self.distance_bias.is_contiguous(),
+                  "distance_bias: a contiguous row a head")
+            t.dist_bias, t.n_dist = _ptr(self.distance_bias), self.distance_bias.shape[1]
+        return t
 
     def args(self, q, n_heads):
         for name in ("head_scale", "slopes"):
@@ -1193,19 +1218,25 @@ def attention_head_dim(columns):
     raise ValueError(f"heads of {columns} columns: the attention kernels take at most {FAST_HEAD_DIMS[-1]}")
 
 
-def attend(ctx, out, q, cache, n_heads, n_kv_heads, head_dim, scale, window=0):
+def attend(ctx, out, q, cache, n_heads, n_kv_heads, head_dim, scale, window=0, terms=None):
     """Causal attention of the step's queries ``q`` ``[tokens, n_heads * head_dim]`` over the pages
     of ``cache`` (a ``CacheView``), into ``out``: the native host chooses among the attention kernels
     as it does for the built-in attention part (single rows to the decode kernels, portions to the
     tile kernels), by the step arrays that part declares (``parts.attention.CausalSelfAttention``:
-    a mixer that calls this names the same ``step_arrays_key``)."""
+    a mixer that calls this names the same ``step_arrays_key``).  ``terms``: ``ScoreTerms``."""
     from ..parts.attention import CausalSelfAttention as A
 
     base = native.array_ids(A.step_arrays_key, A.step_array_names)
     qm, om = native.mat(q), native.mat(out)
+    t = terms.struct(q, n_heads) if terms is not None else None
     with ctx.enter():
-        rc = native.lib().eng_attend(ctypes.byref(ctx.c), ctypes.byref(om), ctypes.byref(qm), cache.slot, int(n_heads),
-                                     int(n_kv_heads), int(head_dim), int(window), float(scale), base)
+        if t is None:
+            rc = native.lib().eng_attend(ctypes.byref(ctx.c), ctypes.byref(om), ctypes.byref(qm), cache.slot, int(n_heads),
+                                         int(n_kv_heads), int(head_dim), int(window), float(scale), base)
+        else:
+            rc = native.lib().eng_attend_terms(ctypes.byref(ctx.c), ctypes.byref(om), ctypes.byref(qm), cache.slot,
+                                               int(n_heads), int(n_kv_heads), int(head_dim), int(window), float(scale),
+                                               base, ctypes.byref(t))
     native.check(rc, "attend")
     return out
 
@@ -1273,9 +1304,10 @@ def gated_group_rmsnorm(out, y, z, weight, groups, eps):
 # experts chosen per token (csrc/experts.hip)
 
 
-def router_choice(idx, weight, z, correction, top):
+def router_choice(idx, weight, z, correction, top, renormalize=False, weight_scale=1.0):
     """From float32 router outputs ``z`` ``[tokens, outputs]``: softmax, the ``top`` largest of
-    softmax + ``correction`` into ``idx`` (int32 ``[tokens, top]``), their softmax values into ``weight``."""
+    softmax + ``correction`` into ``idx`` (int32 ``[tokens, top]``), their softmax values into
+    ``weight``; with ``renormalize`` divided by their sum (+ 1e-20); times ``weight_scale``."""
     lib = build.load("experts")
     ldz = _f32_rows(z, "z", 1)
     T, n_out = z.shape
@@ -1285,12 +1317,12 @@ def router_choice(idx, weight, z, correction, top):
     if correction is not None:
         _dev(correction, "correction", torch.float32)
         _need(correction.numel() == n_out, "router_choice: correction length")
-    rc = lib.router_choice(_ptr(z), _c_int(ldz), _ptr(correction), _c_int(T), _c_int(n_out), _c_int(top), _ptr(idx),
-                           _ptr(weight), _stream())
+    rc = lib.router_choice_scaled(_ptr(z), _c_int(ldz), _ptr(correction), _c_int(T), _c_int(n_out), _c_int(top), _ptr(idx),
+                                  _ptr(weight), _c_int(int(bool(renormalize))), _c_float(weight_scale), _stream())
     build.check(lib, rc, "router_choice")
 
 
-def route_and_gate(idx, weight, act, zu, correction, top, n_out):
+def route_and_gate(idx, weight, act, zu, correction, top, n_out, renormalize=False, weight_scale=1.0):
     """``router_choice`` on the first ``n_out`` columns of the float32 rows ``zu`` and ``silu_mul`` on
     the ``2 * act.shape[1]`` columns behind them, in one launch (for steps of few tokens)."""
     lib = build.load("experts")
@@ -1303,18 +1335,25 @@ def route_and_gate(idx, weight, act, zu, correction, top, n_out):
     if correction is not None:
         _dev(correction, "correction", torch.float32)
         _need(correction.numel() == n_out, "route_and_gate: correction length")
-    rc = lib.route_and_gate(_ptr(zu), _c_int(ld), _ptr(correction), _c_int(T), _c_int(n_out), _c_int(top), _c_int(F),
-                            _ptr(idx), _ptr(weight), _ptr(act), _c_int(ldo), _c_int(DT[act.dtype]), _stream())
+    rc = lib.route_and_gate_scaled(_ptr(zu), _c_int(ld), _ptr(correction), _c_int(T), _c_int(n_out), _c_int(top), _c_int(F),
+                                   _ptr(idx), _ptr(weight), _ptr(act), _c_int(ldo), _c_int(DT[act.dtype]),
+                                   _c_int(int(bool(renormalize))), _c_float(weight_scale), _stream())
     build.check(lib, rc, "route_and_gate")
 
 
-def silu_mul(out, gate_up):
-    """``out = silu(gate_up[:, :F]) * gate_up[:, F:2F]`` with ``F = out.shape[1]``."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def silu_mul(out, gate_up, activation="silu"):
+    """``out = act(gate_up[:, :F]) * gate_up[:, F:2F]`` with ``F = out.shape[1]``; ``activation``:
+    ``silu``, or ``gelu_tanh`` (``0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))``)."""
     lib = build.load("experts")
     ld, ldo = _rows2d(gate_up, "gate_up"), _rows2d(out, "out")
     T, F = out.shape
     _need(gate_up.dtype == out.dtype and out.dtype in DT and gate_up.shape[1] == 2 * F and gate_up.shape[0] >= T, "silu_mul: shapes")
-    rc = lib.silu_mul(_ptr(gate_up), _c_int(ld), _ptr(out), _c_int(ldo), _c_int(T), _c_int(F), _c_int(DT[out.dtype]), _stream())
+    _need(activation in GATE_ACTIVATIONS, f"silu_mul: activation {activation!r} (known: {sorted(GATE_ACTIVATIONS)})")
+    rc = lib.act_mul(_ptr(gate_up), _c_int(ld), _ptr(out), _c_int(ldo), _c_int(T), _c_int(F), _c_int(DT[out.dtype]),
+                     _c_int(GATE_ACTIVATIONS[activation]), _stream())
     build.check(lib, rc, "silu_mul")
     return out
 
@@ -1378,3 +1417,82 @@ def expert_tiles(y, x, w_gate, w_up, w_down, idx, weight, top, alloc, accumulate
                           _stream())
     build.check(lib, rc, "expert_tiles")
     return y
+
+
+# ---------------------------------------------------------------------------
+# a layer whose sublayers share one norm and whose outgoing stream is a sum over depth (csrc/parallel_block.hip)
+
+
+def norm_fanout(out, x, weight, eps, out32=None, copy_a=None, copy_b=None):
+    """``out = x / sqrt(mean(x^2) + eps) * weight`` over the float32 rows ``x`` (``out``: float32 or
+    bfloat16, contiguous); the same as float32 into ``out32``, and ``x`` itself into ``copy_a`` and
+    ``copy_b`` (contiguous float32 ``[rows, width]``), each where given."""
+    lib = build.load("parallel_block")
+    n, width = out.shape
+    ldx = _f32_rows(x, "x", width)
+    _dev(weight, "weight", torch.float32)
+    _need(out.is_contiguous() and out.dtype in DT and weight.numel() == width and x.shape[0] >= n, "norm_fanout: shapes")
+    for name, t in (("out32", out32), ("copy_a", copy_a), ("copy_b", copy_b)):
+        if t is not None:
+            _dev(t, name, torch.float32)
+            _need(t.is_contiguous() and tuple(t.shape) == (n, width), f"norm_fanout: {name} is contiguous [rows, width]")
+    rc = lib.norm_fanout(_ptr(x), _c_int(ldx), _ptr(weight), _c_float(eps), _c_int(n), _c_int(width), _ptr(out),
+                         _c_int(DT[out.dtype]), _ptr(out32), _ptr(copy_a), _ptr(copy_b), _stream())
+    build.check(lib, rc, "norm_fanout")
+    return out
+
+
+def depth_average(out, kept, weights, n):
+    """``out[t] = sum over j < n of weights[j] * kept[j, t]``: ``kept`` float32 ``[>= n, rows, width]``,
+    ``weights`` float32 on the device, ``out`` contiguous float32 ``[rows, width]``."""
+    lib = build.load("parallel_block")
+    _dev(out, "out", torch.float32)
+    _dev(kept, "kept", torch.float32)
+    _dev(weights, "weights", torch.float32)
+    _need(kept.dim() == 3 and kept.shape[0] >= n and kept.is_contiguous() and out.is_contiguous()
+          and tuple(kept.shape[1:]) == tuple(out.shape) and weights.numel() >= n, "depth_average: shapes")
+    rc = lib.depth_average(_ptr(out), _ptr(kept), _c_size_t(kept.stride(0)), _ptr(weights), _c_int(n), _c_int(out.shape[0]),
+                           _c_int(out.shape[1]), _stream())
+    build.check(lib, rc, "depth_average")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# between a projection's float rows and a recurrence, and behind it (csrc/state_gates.hip)
+
+
+def silu_columns(u, col, n):
+    """``u[:, col:col + n] <- silu(...)`` in place on float32 rows."""
+    lib = build.load("state_gates")
+    ld = _f32_rows(u, "u", col + n)
+    rc = lib.silu_columns(_ptr(u), _c_int(ld), _c_int(u.shape[0]), _c_int(col), _c_int(n), _stream())
+    build.check(lib, rc, "silu_columns")
+    return u
+
+
+def forget_gate(u, q_col, z_col, n, lower, keys):
+    """A forget gate with a floor, ``f = lower + (1 - lower) * sigmoid(z)``, for ``S <- diag(f) S +
+    (1 - f) v^T``: the logits ``u[:, z_col:z_col + n]`` become ``log f`` in place, ``1 - f`` goes to
+    ``keys`` (float32 ``[rows, >= n]``), and the queries ``u[:, q_col:q_col + n]`` pass a silu in place."""
+    lib = build.load("state_gates")
+    ld, ldk = _f32_rows(u, "u", max(q_col, z_col) + n), _f32_rows(keys, "keys", n)
+    _dev(lower, "lower", torch.float32)
+    _need(lower.numel() == n and keys.shape[0] >= u.shape[0], "forget_gate: a floor a channel, a row of keys a row")
+    rc = lib.forget_gate(_ptr(u), _c_int(ld), _c_int(u.shape[0]), _c_int(q_col), _c_int(z_col), _c_int(n), _ptr(lower),
+                         _ptr(keys), _c_int(ldk), _stream())
+    build.check(lib, rc, "forget_gate")
+    return keys
+
+
+def normed_gate(out, y, gate, weight, eps):
+    """``out = y / sqrt(mean(y^2) + eps) * weight * sigmoid(gate)`` over whole float32 rows; ``out``
+    float32 or bfloat16 ``[rows, width]`` (its rows may be wider apart)."""
+    lib = build.load("state_gates")
+    n, width = out.shape
+    ldy, ldg, ldo = _f32_rows(y, "y", width), _f32_rows(gate, "gate", width), _rows2d(out, "out")
+    _dev(weight, "weight", torch.float32)
+    _need(out.dtype in DT and weight.numel() == width and y.shape[0] >= n and gate.shape[0] >= n, "normed_gate: shapes")
+    rc = lib.normed_gate(_ptr(y), _c_int(ldy), _ptr(gate), _c_int(ldg), _ptr(weight), _c_float(eps), _c_int(n), _c_int(width),
+                         _ptr(out), _c_int(ldo), _c_int(DT[out.dtype]), _stream())
+    build.check(lib, rc, "normed_gate")
+    return out

@@ -169,6 +169,8 @@ def lib():
         "eng_ffn_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngValue), POINTER(EngMat)]),
         "eng_attend": (c_int, [POINTER(EngCtx), POINTER(EngMat), POINTER(EngMat), c_int, c_int, c_int, c_int, c_int,
                                c_float, c_int]),
+        "eng_attend_terms": (c_int, [POINTER(EngCtx), POINTER(EngMat), POINTER(EngMat), c_int, c_int, c_int, c_int, c_int,
+                                     c_float, c_int, P]),
         "eng_embedding_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngMat), P]),
         "eng_head_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngValue), POINTER(EngMat)]),
         "eng_settle": (c_int, [POINTER(EngCtx)]),

@@ -1,7 +1,7 @@
 """Parts that models are put together from; importing this registers the built-in kinds."""
 
 from . import (attention, block, convolution, differential_attention, embedding, experts, feed_forward,  # noqa: F401
-               gated_attention, head, latent_attention, linear_state, norms, positions)
+               gated_attention, head, latent_attention, linear_state, norms, positions, scored_attention)
 from .base import (
     BLOCKS,
     EMBEDDINGS,

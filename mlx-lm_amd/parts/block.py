@@ -232,6 +232,130 @@ class SandwichBlock(Block):
         return h
 
 
+class SharedNormBlock(Block):
+    """``y = h + mixer(u + conv(u)) + ffn(u)`` with ``u = norm(h)``: one norm, which both sublayers
+    read, and their outputs enter the stream together.  Two options around it:
+
+    * ``input_taps``: what the mixer reads passes a causal convolution over time on each channel
+      first and is added to itself, ``u_t + sum_j w[:, j] u_(t - taps + 1 + j)`` (tensor
+      ``input_conv_name``, ``[width, taps]``, no bias, zeros before a request's start); the
+      feed-forward reads ``u`` as it is.  The last ``taps - 1`` normed rows are the request's state.
+    * ``depth``: the stream that leaves the layer is a weighted sum over depth, ``h <- sum_(j <=
+      depth + 1) a[j] Y_j`` with ``Y_0`` the stream as the first layer found it, ``Y_(i+1)`` the
+      ``y`` of the layer with ``depth = i``, and ``a`` the tensor ``depth_name`` (``depth + 2``
+      values).  The layers of a step share the ``Y`` through ``ctx.shared`` (``depth_total``
+      layers: the one with ``depth = 0`` takes the memory, the sublayers add straight into ``Y``).
+
+    The norm is an RMS norm (an ``rmsnorm`` part gives weight and eps).  Norm, convolution, the
+    sums and the weighted sum are 32-bit (csrc/parallel_block.hip, csrc/head_prepare.hip).  The
+    run's state slot holds the convolution's inputs and, behind them, what a mixer that keeps
+    state beside its pages (``wants_state``) asks for.  No counterpart in mlx_lm/models/gpt2.py,
+    whose blocks have a norm for each sublayer and run them in turn (:98-108).
+    """
+
+    PARTS = {"norm": "norm", "mixer": "mixer", "ffn": "feed_forward"}
+    OPTIONAL = ("ffn",)
+
+    def __init__(self, norm, mixer, ffn=None, input_taps=0, input_conv_name="canon1", depth=None, depth_total=0,
+                 depth_name="dwa", prefix=""):
+        from .convolution import ShortConvolution
+
+        super().__init__(prefix)
+        if not (hasattr(norm, "weight") and hasattr(norm, "eps")) or hasattr(norm, "bias"):
+            raise ValueError(f"this arrangement fuses an RMS norm, not a {type(norm).__name__}")
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+        self.width, self.eps = norm.width, norm.eps
+        if self.width % 8:
+            raise ValueError(f"width {self.width} must be a multiple of 8")
+        self.input_conv = ShortConvolution((self.width,), int(input_taps), (input_conv_name,), add_identity=True,
+                                           prefix=prefix) if input_taps else None
+        # (the convolution runs as ``head_prepare`` reads a row in pieces of at most 256 columns)
+        self.conv_piece = next(d for d in (256, 128, 64, 32, 16, 8) if self.width % d == 0)
+        if depth is not None and not 0 <= depth < depth_total:
+            raise ValueError(f"depth {depth} of {depth_total} layers")
+        self.depth, self.depth_total, self.depth_name = depth, int(depth_total), self._name(depth_name)
+        self.depth_w = None
+        self.conv_floats = self.input_conv.state_floats if self.input_conv is not None else 0
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.parts() if p is not self)
+
+    def parts(self):
+        out = []
+
+        def walk(part):
+            if part is None:
+                return
+            out.append(part)
+            for sub in getattr(part, "sub_parts", lambda: ())():
+                walk(sub)
+
+        for p in (self.norm, self.input_conv, self.mixer, self.ffn):
+            walk(p)
+        return tuple(out) + (self,)  # (the arrangement owns a tensor itself, so it is one of its own parts)
+
+    def tensors(self):
+        return {self.depth_name: TensorSpec((self.depth + 2,), "vector")} if self.depth is not None else {}
+
+    def load(self, tensors):
+        if self.depth is not None:
+            self.depth_w = tensors[self.depth_name].contiguous()
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def _mixer_state_need(self):
+        if getattr(self.mixer, "wants_state", False) and hasattr(self.mixer, "state_need"):
+            return self.mixer.state_need()
+        return None
+
+    def state_need(self):
+        need, floats = self._mixer_state_need(), self.conv_floats
+        if need is not None:
+            if need.dtype != "float32" or len(need.shape) != 1:
+                raise ValueError("a mixer's state beside its pages is a row of float32")
+            floats += need.shape[0]
+        return StateNeed((floats,), "float32") if floats else None
+
+    def forward(self, ctx, h, cache, writes_cache=True, state=None):
+        import torch
+
+        from ..engine.context import CacheView
+        from ..ops import kernels
+
+        T, W = h.shape
+        kept = target = None
+        if self.depth is not None:
+            if self.depth == 0:
+                # every layer's result of this step, the stream as it came first: kept to the step's end
+                ctx.shared["depth_results"] = ctx.scratch((self.depth_total + 1, T, W), torch.float32)
+            kept = ctx.shared["depth_results"]
+            target = kept[self.depth + 1]
+        mark = ctx.scratch_mark()
+        u = ctx.scratch((T, W), ctx.dtype)
+        u32 = ctx.scratch((T, W), torch.float32) if self.input_conv is not None else None
+        # the norm; the stream itself goes where the sublayers add to it (and, first of all, to Y_0)
+        kernels.norm_fanout(u, h, self.norm.weight, self.eps, out32=u32, copy_a=target,
+                            copy_b=kept[0] if self.depth == 0 else None)
+        um = u
+        if self.input_conv is not None:
+            um = ctx.scratch((T, W), ctx.dtype)
+            rows = state.state if state is not None else None
+            kernels.head_prepare(um, u32, 0, W // self.conv_piece, self.conv_piece, conv=self.input_conv.ahead(ctx, rows, 0))
+            self.input_conv.keep_inputs(ctx, u32, rows, 0)
+        into = target if target is not None else h
+        if self._mixer_state_need() is not None:
+            self.mixer.forward(ctx, um, into, cache, writes_cache,
+                               state=CacheView(state.slot, state=state.state, offset=self.conv_floats))
+        else:
+            self.mixer.forward(ctx, um, into, cache, writes_cache)
+        if self.ffn is not None:
+            self.ffn.forward(ctx, u, into)
+        ctx.scratch_release(mark)
+        if kept is not None:
+            kernels.depth_average(h, kept, self.depth_w, self.depth + 2)
+        return h
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("shared_norm", SharedNormBlock)
 register_block("sandwich", SandwichBlock)
 register_block("post_norm", PostNormBlock)

@@ -13,8 +13,8 @@ class GatedExperts(FeedForward):
       ``e<i>.gate``, ``e<i>.up`` (``[inner, width]``) and ``e<i>.down`` (``[width, inner]``);
     * ``s = softmax(Wrouter x)`` over all ``n_experts + n_identity`` router outputs (32-bit sums
       of the products of the compute dtype's operands); the ``top`` largest of ``s + correction``
-      are chosen (``correction``: a tensor, or none), and weigh in with ``s`` itself, not
-      renormalised;
+      are chosen (``correction``: a tensor, or none), and weigh in with ``s`` itself; with
+      ``renormalize`` divided by the chosen ones' sum (+ 1e-20); times ``weight_scale``;
     * the last ``n_identity`` router outputs stand for experts that give their input back;
     * ``shared_inner > 0``: one more expert of that inner size (``shared.gate`` ...) that every
       token uses with weight one.
@@ -32,8 +32,10 @@ class GatedExperts(FeedForward):
     MERGED_UP_TO = 16  # up to this many tokens the router's and the shared expert's first products are one
     TILES_FROM = 64  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
 
-    def __init__(self, width, n_experts, inner, top, n_identity=0, shared_inner=0, correction=True, prefix=""):
+    def __init__(self, width, n_experts, inner, top, n_identity=0, shared_inner=0, correction=True, renormalize=False,
+                 weight_scale=1.0, prefix=""):
         super().__init__(prefix)
+        self.renormalize, self.weight_scale = bool(renormalize), float(weight_scale)
         if n_experts < 0 or n_identity < 0 or n_experts + n_identity <= 0:
             raise ValueError(f"{n_experts} experts and {n_identity} identity experts")
         if not 0 < top <= n_experts + n_identity:
@@ -97,13 +99,13 @@ class GatedExperts(FeedForward):
             zu = ctx.scratch((T, self.n_out + 2 * self.shared_padded), torch.float32)
             kernels.linear(zu, x, self.merged_in)
             act = ctx.scratch((T, self.shared_padded), ctx.dtype)
-            kernels.route_and_gate(idx, weight, act, zu, self.correction, self.top, self.n_out)
+            kernels.route_and_gate(idx, weight, act, zu, self.correction, self.top, self.n_out, self.renormalize, self.weight_scale)
             kernels.linear(residual, act, self.shared_out, accumulate=accumulate)
             accumulate = True
         else:
             z = ctx.scratch((T, self.n_out), torch.float32)
             kernels.linear(z, x, self.router_w, splits=kernels.splits_alone(T))
-            kernels.router_choice(idx, weight, z, self.correction, self.top)
+            kernels.router_choice(idx, weight, z, self.correction, self.top, self.renormalize, self.weight_scale)
         if self.shared_inner and T > self.MERGED_UP_TO:
             gu = ctx.scratch((T, 2 * self.shared_padded), ctx.dtype)
             kernels.linear(gu, x, self.shared_in, splits=kernels.splits_alone(T))

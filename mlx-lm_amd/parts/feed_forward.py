@@ -119,7 +119,7 @@ class Relu2MLP(FeedForward):
 
 
 class GatedMLP(FeedForward):
-    """``down(silu(gate(x)) * up(x))``, dense, no biases.
+    """``down(act(gate(x)) * up(x))``, dense, no biases; ``activation``: ``silu`` or ``gelu_tanh``.
 
     One product gives ``[gate | up]``; the activation and the product of the two halves are one
     kernel (``silu_mul``, which the experts' shared expert uses too); the second product adds into
@@ -129,8 +129,11 @@ class GatedMLP(FeedForward):
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
     takes_normed_input = True  # ``x`` may be a ``kernels.NormedInput``: the first product norms the rows itself
 
-    def __init__(self, width, inner, gate_name="gate", up_name="up", down_name="down", prefix=""):
+    def __init__(self, width, inner, gate_name="gate", up_name="up", down_name="down", activation="silu", prefix=""):
         super().__init__(prefix)
+        if activation not in kernels.GATE_ACTIVATIONS:
+            raise ValueError(f"gate activation {activation!r} is not implemented (known: {sorted(kernels.GATE_ACTIVATIONS)})")
+        self.activation = activation
         if width % 8:
             raise ValueError(f"the feed-forward's width must be a multiple of 8, got {width}")
         if inner <= 0:
@@ -162,7 +165,7 @@ class GatedMLP(FeedForward):
         gate_up = ctx.scratch((T, 2 * F), ctx.dtype)
         kernels.linear(gate_up, x, self.gate_up_w, splits=kernels.splits_alone(T))
         act = ctx.scratch((T, F), ctx.dtype)
-        kernels.silu_mul(act, gate_up)
+        kernels.silu_mul(act, gate_up, self.activation)
         kernels.linear(residual, act, self.down_w, accumulate=True, splits=kernels.splits_alone(T))
         ctx.scratch_release(mark)
 

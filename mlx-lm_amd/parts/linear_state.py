@@ -305,6 +305,139 @@ class StateSpace(_SequenceArrays, Mixer):
         ctx.scratch_release(mark)
 
 
+class LightningAttention(_SequenceArrays, Mixer):
+    """Linear attention with a fixed decay per head, activated projections and one norm over all heads:
+
+        ``S_t = decay_h S_(t-1) + k_t v_t^T``,   ``o_t = S_t^T q_t``
+
+    with ``q = silu(Wq x)``, ``k = silu(Wk x)`` (``n_heads x key_dim``), ``v = silu(Wv x)`` (``n_heads x
+    value_dim``) and no other scale.  The concatenated heads are RMS-normed together with the weight
+    ``norm`` (``n_heads * value_dim`` values), multiplied by ``sigmoid(Wg x)`` and projected by
+    ``Wo``.  ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start) is the
+    request's state.  One product gives ``[q | k | v | g]`` as float32 rows; the activations, the
+    recurrence, the norm and the gate are 32-bit (csrc/state_gates.hip, csrc/linear_state.hip).
+    No counterpart in mlx_lm/models/gpt2.py.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, width, n_heads, key_dim, value_dim, decay, eps, prefix=""):
+        super().__init__(prefix)
+        if n_heads <= 0 or key_dim <= 0 or not 0 < value_dim <= 256:
+            raise ValueError(f"{n_heads} heads of keys {key_dim} and values {value_dim} (values at most 256)")
+        if len(decay) != n_heads or any(not 0.0 < float(d) <= 1.0 for d in decay):
+            raise ValueError(f"decays {list(decay)}: one in (0, 1] for each of the {n_heads} heads")
+        if width % 8:
+            raise ValueError(f"width {width} must be a multiple of 8")
+        self.width, self.n_heads, self.key_dim, self.value_dim = width, n_heads, key_dim, value_dim
+        self.decay_values, self.eps = [float(d) for d in decay], float(eps)
+        self.qk_width, self.v_width = n_heads * key_dim, n_heads * value_dim
+
+    def cache_need(self):
+        return StateNeed((self.n_heads * self.key_dim * self.value_dim,), "float32")
+
+    def tensors(self):
+        n = self._name
+        return {n("q"): TensorSpec((self.qk_width, self.width), "matrix"),
+                n("k"): TensorSpec((self.qk_width, self.width), "matrix"),
+                n("v"): TensorSpec((self.v_width, self.width), "matrix"),
+                n("g"): TensorSpec((self.v_width, self.width), "matrix"),
+                n("o"): TensorSpec((self.width, self.v_width), "matrix"),
+                n("norm"): TensorSpec((self.v_width,), "vector")}
+
+    def load(self, tensors):
+        n = self._name
+        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in ("q", "k", "v", "g")]))
+        self.out_w = _matrix(_padded_columns(tensors[n("o")]))
+        self.first_weight = self.in_w
+        self.norm_w = tensors[n("norm")]
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=self.norm_w.device)
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True):
+        T = x.shape[0]
+        mark = ctx.scratch_mark()
+        a, b = self.qk_width, 2 * self.qk_width
+        u = ctx.scratch((T, b + 2 * self.v_width), torch.float32)
+        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
+        kernels.silu_columns(u, 0, b + self.v_width)
+        y = ctx.scratch((T, self.v_width), torch.float32)
+        kernels.state_scan(y, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, cache.offset,
+                           ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,
+                           self.n_heads, self.n_heads, self.key_dim, self.value_dim, decay=self.decay,
+                           chunked=self._chunked(ctx), spans=self._spans(ctx))
+        out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
+        kernels.normed_gate(out, y, u[:, b + self.v_width:], self.norm_w, self.eps)
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=True, splits=kernels.splits_alone(T))
+        ctx.scratch_release(mark)
+
+
+class ForgetGateAttention(_SequenceArrays, Mixer):
+    """Linear attention in which the forget gate also decides what is written (HGRN2):
+
+        ``S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T``,   ``o_t = S_t^T q_t``
+
+    with ``q = silu(Wq x)`` (``n_heads x key_dim``), ``v = Wv x`` (``n_heads x value_dim``) and, per
+    head and key channel, ``f = l + (1 - l) sigmoid(Wf x + b)`` with the floor ``l`` from the tensor
+    ``lower``; there is no key projection and no other scale.  Each head's ``o`` is RMS-normed over
+    ``value_dim`` with the weight ``norm`` (shared by the heads), the heads are concatenated and
+    projected by ``Wo``.  ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start)
+    is the request's state.  One product gives ``[q | z | v]`` as float32 rows; ``1 - f`` (made as
+    ``(1 - l) sigmoid(-z)``, without cancellation), ``log f``, the recurrence with a decay per key
+    channel and the norm are 32-bit (csrc/state_gates.hip, csrc/linear_state.hip).  No counterpart
+    in mlx_lm/models/gpt2.py.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, width, n_heads, key_dim, value_dim, eps, prefix=""):
+        super().__init__(prefix)
+        if n_heads <= 0 or key_dim <= 0 or not 0 < value_dim <= 256:
+            raise ValueError(f"{n_heads} heads of keys {key_dim} and values {value_dim} (values at most 256)")
+        if width % 8:
+            raise ValueError(f"width {width} must be a multiple of 8")
+        self.width, self.n_heads, self.key_dim, self.value_dim, self.eps = width, n_heads, key_dim, value_dim, float(eps)
+        self.qk_width, self.v_width = n_heads * key_dim, n_heads * value_dim
+
+    def cache_need(self):
+        return StateNeed((self.n_heads * self.key_dim * self.value_dim,), "float32")
+
+    def tensors(self):
+        n = self._name
+        return {n("q"): TensorSpec((self.qk_width, self.width), "matrix"),
+                n("f"): TensorSpec((self.qk_width, self.width), "matrix"),
+                n("f.b"): TensorSpec((self.qk_width,), "vector"),
+                n("lower"): TensorSpec((self.qk_width,), "vector"),
+                n("v"): TensorSpec((self.v_width, self.width), "matrix"),
+                n("norm"): TensorSpec((self.value_dim,), "vector"),
+                n("o"): TensorSpec((self.width, self.v_width), "matrix")}
+
+    def load(self, tensors):
+        n = self._name
+        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in ("q", "f", "v")]))
+        bias = tensors[n("f.b")]
+        self.in_b = torch.cat([bias.new_zeros(self.qk_width), bias, bias.new_zeros(self.v_width)]).contiguous()
+        self.first_weight = self.in_w
+        self.out_w = _matrix(_padded_columns(tensors[n("o")]))
+        self.lower, self.norm_w = tensors[n("lower")].contiguous(), tensors[n("norm")]
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True):
+        T = x.shape[0]
+        mark = ctx.scratch_mark()
+        a, b = self.qk_width, 2 * self.qk_width
+        u = ctx.scratch((T, b + self.v_width), torch.float32)
+        kernels.linear(u, x, self.in_w, bias=self.in_b, splits=kernels.splits_alone(T))
+        keys = ctx.scratch((T, a), torch.float32)
+        kernels.forget_gate(u, 0, a, a, self.lower, keys)  # (queries activated, logits to log f, keys = 1 - f)
+        out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
+        kernels.state_scan(out, u[:, :a], keys, u[:, b:], cache.state, cache.offset,
+                           ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,
+                           self.n_heads, self.n_heads, self.key_dim, self.value_dim, channel_decay=u[:, a:b],
+                           unit_rms=True, eps=self.eps, norm_weight=self.norm_w, chunked=self._chunked(ctx),
+                           spans=self._spans(ctx))
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=True, splits=kernels.splits_alone(T))
+        ctx.scratch_release(mark)
+
+
 class ParallelMixers(Mixer):
     """Two mixers side by side that read the same input: ``left_scale * left(x) + right_scale *
     right(x)``.  The left one keeps the run's cache slot, the right one the run's state slot (the
@@ -358,4 +491,6 @@ class ParallelMixers(Mixer):
 register_mixer("retention", Retention)
 register_mixer("gated_linear_attention", GatedLinearAttention)
 register_mixer("state_space", StateSpace)
+register_mixer("lightning_attention", LightningAttention)
+register_mixer("forget_gate_attention", ForgetGateAttention)
 register_mixer("parallel", ParallelMixers)

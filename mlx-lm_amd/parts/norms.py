@@ -59,6 +59,7 @@ class LayerNorm(Norm):
 
 class RMSNorm(Norm):
     """``x / sqrt(mean(x^2) + eps) * weight``: no mean is taken off, eps sits inside the root.
+    With ``offset`` the scale is ``offset + weight`` (a weight stored around zero with ``offset = 1``).
 
     Reads the float32 residual stream, computes in float32, writes the compute dtype (``rows``:
     only those rows, for the rows whose logits are wanted).  An arrangement that norms after
@@ -68,11 +69,11 @@ class RMSNorm(Norm):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
 
-    def __init__(self, width, eps, weight_name="weight", prefix=""):
+    def __init__(self, width, eps, weight_name="weight", offset=0.0, prefix=""):
         super().__init__(prefix)
         if eps < 0:
             raise ValueError(f"eps must not be negative, got {eps}")
-        self.width, self.eps = width, float(eps)
+        self.width, self.eps, self.offset = width, float(eps), float(offset)
         self.weight_name = self._name(weight_name)
         self.weight = None
 
@@ -80,7 +81,8 @@ class RMSNorm(Norm):
         return {self.weight_name: TensorSpec((self.width,), "vector")}
 
     def load(self, tensors):
-        self.weight = tensors[self.weight_name]
+        # ``offset``: the tensor is stored around zero and the scale is ``offset + tensor`` (float32)
+        self.weight = tensors[self.weight_name] + self.offset if self.offset else tensors[self.weight_name]
 
     def make_native(self):
         L = native.part_library("rmsnorm", {"make_rmsnorm": [ctypes.c_int, ctypes.c_float, ctypes.c_void_p]})
