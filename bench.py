@@ -35,7 +35,8 @@ Pafutar model runs once without a window (like for like with GPT-2's attention) 
 window of 512 that keeps the first 64 tokens.  Ruzolorn runs at the same layer sizes too
 (``ruzolorn_config``), without a window and with one of 512, and Zatinex (``zatinex_config``:
 differential attention, gated linear attention and latent attention by turns, a dense gated
-feed-forward).  It prints one JSON line of its own.
+feed-forward), and Sazilorn (``sazilorn_config``: its parallel, HGRN2 and attention mixers by turns,
+dense and expert feed-forwards).  It prints one JSON line of its own.
 """
 
 import argparse
@@ -75,6 +76,8 @@ def design_config(design, size, window=None):
         return ruzolorn_config(s, window)
     if design == "zatinex":
         return zatinex_config(s)
+    if design == "sazilorn":
+        return sazilorn_config(s)
     mixer = {"heads": s["heads"], "kv_heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5}
     if window:
         mixer["mask"] = {"size": window[0], "keep_first": window[1]}
@@ -142,6 +145,30 @@ def zatinex_config(s):
             "norm": {"eps": 1e-5}, "layers": layers}
 
 
+def sazilorn_config(s):
+    """Sazilorn at GPT-2's layer sizes, its three mixers by turns, four taps ahead of every mixer and
+    the sum over depth behind every layer.  Parallel: capped, gated softmax attention with as many
+    heads of the same size over a quarter as many key heads, beside lightning attention with half
+    as many heads.  HGRN2: as many heads of the same size (Zatinex's gated linear attention and
+    Ruzolorn's retention at the same sizes are its like).  Attention: grouped key heads as above,
+    whole-projection norms, a distance table of 32 rows reaching to 128.  Feed-forwards by turns: a
+    gelu-gated dense one of two thirds of GPT-2's inner size, and Ruzolorn's mixture at its sizes
+    (sixteen experts of an eighth, four a token, a shared expert of a quarter)."""
+    H, d, D = s["heads"], s["dim"], s["width"]
+    G = max(1, H // 4)
+    left = {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 30.0}
+    R = max(1, H // 2)
+    right = {"heads": R, "dim": d, "vdim": d, "decay": [1.0 - 2.0 ** (-5.0 - 5.0 * h / max(1, R - 1)) for h in range(R)]}
+    mixers = [("parallel", {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}),
+              ("hgrn2", {"heads": H, "dim": d, "vdim": d}),
+              ("attention", {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5, "bias_rows": 32, "bias_max": 128})]
+    dense = {"kind": "dense", "ff": s["ff"] * 2 // 3 // 64 * 64}
+    moe = {"kind": "moe", "expert": {"ff": s["ff"] // 8}, "router": {"experts": 16, "top": 4, "scale": 2.0}, "shared": {"ff": s["ff"] // 4}}
+    layers = [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": moe if i % 3 == 1 else dense} for i in range(s["layers"])]
+    return {"architecture": "Sazilorn", "vocab": DESIGN_VOCAB, "width": D, "max_positions": DESIGN_POSITIONS,
+            "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "layers": layers}
+
+
 def bench_design(config, dtype, batches, steps, warmup):
     """Prefill of 2 x 1,024 tokens (three warm-up trials, the mean of five) and decode from
     context 512 at each of ``batches``, for the model that ``config`` describes."""
@@ -189,7 +216,7 @@ def compare_designs(a):
     for size in sizes:
         entry = {"layer_sizes": DESIGN_SIZES[size]}
         runs = {"gpt2": ("gpt2", None), "pafutar": ("pafutar", None), "pafutar_window_512_keep_64": ("pafutar", (512, 64)),
-                "ruzolorn": ("ruzolorn", None), "ruzolorn_window_512": ("ruzolorn", (512, 0)), "zatinex": ("zatinex", None)}
+                "ruzolorn": ("ruzolorn", None), "ruzolorn_window_512": ("ruzolorn", (512, 0)), "zatinex": ("zatinex", None), "sazilorn": ("sazilorn", None)}
         for name, (design, window) in runs.items():
             if a.design_only and name != a.design_only:
                 continue
@@ -298,7 +325,7 @@ def main():
     ap.add_argument("--designs", action="store_true",
                     help="a mode of its own: Pafutar beside GPT-2 at equal layer sizes (prefill and decode)")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default=None, help="with --designs: one size only")
-    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64, ruzolorn, ruzolorn_window_512, zatinex")
+    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64, ruzolorn, ruzolorn_window_512, zatinex, sazilorn")
     a = ap.parse_args()
     if a.designs:
         if a.gpus != 1:

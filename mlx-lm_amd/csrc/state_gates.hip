@@ -26,9 +26,10 @@ __global__ __launch_bounds__(256) void forget_gate_kernel(float* __restrict__ u,
   if (c >= n) return;
   float* row = u + (size_t)blockIdx.x * ld;
   const float z = row[z_col + c], l = lower[c];
-  // 1 - f without cancellation; log f = log1p(-(1 - f)) keeps its digits where f is close to one
+  // 1 - f without cancellation; log f = log1p(-(1 - f)) keeps its digits where f is close to one,
+  // log(l + (1 - l) sigmoid(z)) where it is small
   const float rest = (1.0f - l) / (1.0f + expf(z));
-  row[z_col + c] = log1pf(-rest);
+  row[z_col + c] = rest < 0.5f ? log1pf(-rest) : logf(l + (1.0f - l) / (1.0f + expf(-z)));
   keys[(size_t)blockIdx.x * ldk + c] = rest;
   row[q_col + c] = silu_f(row[q_col + c]);
 }

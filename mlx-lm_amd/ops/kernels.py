@@ -635,7 +635,8 @@ class ScoreTerms:
 
 
 def _terms(terms, q, n_heads):
-    return (terms or ScoreTerms()).args(q, n_heads)
+    """The terms as the one argument that the kernels' ``_terms`` entry points take."""
+    return [ctypes.byref((terms or ScoreTerms()).struct(q, n_heads))]
 
 
 def attn_tile(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0, terms=None):
@@ -650,7 +651,7 @@ def attn_tile(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_h
     _attn_common(q, kv, block_table, token_req, positions)
     _dev(tiles, "tiles", torch.int32)
     _need(tiles.numel() >= 2 * n_tiles, "attn_tile: tile list too short")
-    rc = lib.attn_tile_biased(
+    rc = lib.attn_tile_terms(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(tiles), _c_int(n_tiles), _c_int(n_heads),
@@ -681,7 +682,7 @@ def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_head
         _dev(part_ml, "part_ml", torch.float32)
         _need(part_o.numel() >= n_rows * n_heads * n_splits * kv.head_dim, "attn_row: part_o too small")
         _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_row: part_ml too small")
-    rc = lib.attn_row_biased(
+    rc = lib.attn_row_terms(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
@@ -729,7 +730,7 @@ def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, 
     _attn_common(q, kv, block_table, token_req, positions)
     _dev(tiles, "tiles", torch.int32)
     _need(tiles.numel() >= 2 * n_tiles, "attn_prefill: tile list too short")
-    rc = lib.attn_prefill_biased(
+    rc = lib.attn_prefill_terms(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(tiles), _c_int(n_tiles), _c_int(n_heads),
@@ -778,7 +779,7 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_decode: part_ml too small")
     if rows_are_requests:
         _need(n_rows <= block_table.shape[0], "attn_decode: more rows than requests")
-    rc = lib.attn_decode_rows_biased(
+    rc = lib.attn_decode_rows_terms(
         _ptr(out.data if packed_out else out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),

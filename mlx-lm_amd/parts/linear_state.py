@@ -320,6 +320,7 @@ class LightningAttention(_SequenceArrays, Mixer):
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
+    can_overwrite = True  # writes its output instead of adding it where ``overwrite`` is set
 
     def __init__(self, width, n_heads, key_dim, value_dim, decay, eps, prefix=""):
         super().__init__(prefix)
@@ -332,6 +333,7 @@ class LightningAttention(_SequenceArrays, Mixer):
         self.width, self.n_heads, self.key_dim, self.value_dim = width, n_heads, key_dim, value_dim
         self.decay_values, self.eps = [float(d) for d in decay], float(eps)
         self.qk_width, self.v_width = n_heads * key_dim, n_heads * value_dim
+        self.overwrite = False
 
     def cache_need(self):
         return StateNeed((self.n_heads * self.key_dim * self.value_dim,), "float32")
@@ -367,7 +369,7 @@ class LightningAttention(_SequenceArrays, Mixer):
                            chunked=self._chunked(ctx), spans=self._spans(ctx))
         out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
         kernels.normed_gate(out, y, u[:, b + self.v_width:], self.norm_w, self.eps)
-        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=True, splits=kernels.splits_alone(T))
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite, splits=kernels.splits_alone(T))
         ctx.scratch_release(mark)
 
 

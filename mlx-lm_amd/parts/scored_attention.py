@@ -47,6 +47,7 @@ class ScoredAttention(Mixer):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
     takes_normed_input = True  # ``x`` may be a ``kernels.NormedInput``: the first product norms the rows itself
+    can_overwrite = True  # writes its output instead of adding it where ``overwrite`` is set
     step_arrays_key = CausalSelfAttention.step_arrays_key
     step_array_names = CausalSelfAttention.step_array_names
     step_arrays = staticmethod(CausalSelfAttention.step_arrays)
@@ -77,6 +78,7 @@ class ScoredAttention(Mixer):
         self.q_cols, self.k_cols, self.v_cols = n_heads * key_dim, n_kv_heads * key_dim, n_kv_heads * value_dim
         self.g_cols = n_heads * value_dim if self.has_gate else 0
         self.distance_bias = None
+        self.overwrite = False
 
     def cache_need(self):
         return CacheNeed(self.n_kv_heads, self.head_dim, self.window)
@@ -140,7 +142,7 @@ class ScoredAttention(Mixer):
             terms = kernels.ScoreTerms(gate=gate, softcap=self.softcap, distance_bias=self.distance_bias)
         att = ctx.scratch((T, H * hd), ctx.dtype)
         kernels.attend(ctx, att, q, cache, H, G, hd, self.scale, self.window, terms=terms)
-        kernels.linear(residual, att, self.out_w, accumulate=True, splits=kernels.splits_alone(T))
+        kernels.linear(residual, att, self.out_w, accumulate=not self.overwrite, splits=kernels.splits_alone(T))
         ctx.scratch_release(mark)
 
 

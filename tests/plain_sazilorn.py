@@ -75,11 +75,9 @@ def grouped_heads(h, w, p, m, normed_eps=None, softcap=0.0, rel=None, far=None):
         g = head // (H // G)
         bias = None
         if rel is not None:
-            rows = rel.shape[0]
-            bias = torch.zeros(T, T, dtype=h.dtype)
-            for i in range(T):
-                for j in range(i + 1):
-                    bias[i, j] = rel[distance_bucket(i - j, rows, far), head]
+            by_distance = torch.stack([rel[distance_bucket(n, rel.shape[0], far), head] for n in range(T)])
+            i = torch.arange(T)
+            bias = by_distance[(i[:, None] - i[None, :]).clamp(min=0)]  # (what lies above the diagonal is masked)
         outs.append(softmax_attention(q[:, head], k[:, g], v[:, g], m["scale"], softcap, bias))
     return torch.cat(outs, -1)
 
@@ -164,11 +162,23 @@ def feed_forward(h, w, p, mlp):
     return experts_ff(h, w, p, mlp)
 
 
+def choice_margin(h, w, p, router):
+    """How far the last chosen expert's choice score lies above the first one left out, per token
+    (infinite where every expert is chosen)."""
+    s = torch.softmax(h @ w[p + "router"].t(), -1) + w[p + "correction"]
+    top = int(router["top"])
+    if top >= s.shape[-1]:
+        return torch.full((h.shape[0],), float("inf"), dtype=h.dtype)
+    ranked = s.sort(-1, descending=True).values
+    return ranked[:, top - 1] - ranked[:, top]
+
+
 MIXERS = {"parallel": parallel_mixer, "hgrn2": hgrn2_mixer, "attention": attention_mixer}
 
 
-def forward(config, w, tokens, return_layers=False):
-    """Logits ``[T, vocab]`` of a whole sequence (and the stream after every layer)."""
+def forward(config, w, tokens, return_layers=False, margins=None):
+    """Logits ``[T, vocab]`` of a whole sequence (and the stream after every layer).  ``margins``: a
+    list that gets every expert layer's ``choice_margin``."""
     eps = float(config["norm"]["eps"])
     T = len(tokens)
     x = w["embed"][torch.tensor(tokens)] + w["pos"][:T]
@@ -180,8 +190,82 @@ def forward(config, w, tokens, return_layers=False):
         y = x + MIXERS[entry["type"]](hm, w, p + "mix.", entry["mixer"], eps)
         if entry.get("mlp") is not None:
             y = y + feed_forward(h, w, p + "mlp.", entry["mlp"])
+            if margins is not None and entry["mlp"]["kind"] == "moe":
+                margins.append(choice_margin(h, w, p + "mlp.", entry["mlp"]["router"]))
         history.append(y)
         x = sum(w[p + "dwa"][j] * history[j] for j in range(i + 2)) if p + "dwa" in w else y
         after.append(x)
     logits = rms_norm(x, 1.0 + w["final.norm"], eps) @ w["head"].t()
     return (logits, torch.stack(after)) if return_layers else logits
+
+
+def random_weights(config, seed, sharp=1.0):
+    """Seeded float32 tensors under the checkpoint's names, every one drawn (norm weights around
+    zero or one as the design stores them).  ``sharp`` multiplies the query and key projections of
+    the softmax attentions, so that their maps are peaked and a key taken wrongly shows."""
+    g = torch.Generator().manual_seed(int(seed))
+    D, taps = config["width"], config["canon"]["taps"]
+
+    def n(shape, std, mean=0.0):
+        return torch.randn(shape, generator=g) * std + mean
+
+    def ff(w, p, F):
+        w[p + "gate"], w[p + "up"], w[p + "down"] = n((F, D), D ** -0.5), n((F, D), D ** -0.5), n((D, F), F ** -0.5)
+
+    def heads(w, p, a):
+        H, G, d, dv = a["heads"], a.get("kv_heads", a["heads"]), a["dim"], a.get("vdim", a["dim"])
+        w[p + "q"], w[p + "k"] = n((H * d, D), D ** -0.5) * sharp, n((G * d, D), D ** -0.5) * sharp
+        w[p + "v"], w[p + "o"] = n((G * dv, D), D ** -0.5), n((D, H * dv), (H * dv) ** -0.5)
+        return H, G, d, dv
+
+    w = {"embed": n((config["vocab"], D), 1.0), "pos": n((config["max_positions"], D), 0.5)}
+    for i, entry in enumerate(config["layers"]):
+        p, m = f"l{i}.", entry["mixer"]
+        w[p + "norm1"], w[p + "canon1"] = n((D,), 0.1), n((D, taps), 0.4)
+        w[p + "dwa"] = n((i + 2,), 0.3, 0.1)
+        w[p + "dwa"][-1] += 0.7
+        q = p + "mix."
+        if entry["type"] == "parallel":
+            H, G, d, dv = heads(w, q + "left.", m["left"])
+            w[q + "left.g"] = n((H * dv, D), D ** -0.5)
+            r = m["right"]
+            H, d, dv = r["heads"], r["dim"], r.get("vdim", r["dim"])
+            for name, rows in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv)):
+                w[q + "right." + name] = n((rows, D), D ** -0.5)
+            w[q + "right.o"], w[q + "right.norm"] = n((D, H * dv), (H * dv) ** -0.5), n((H * dv,), 0.1, 1.0)
+        elif entry["type"] == "hgrn2":
+            H, d, dv = m["heads"], m["dim"], m.get("vdim", m["dim"])
+            w[q + "q"], w[q + "f"], w[q + "v"] = n((H * d, D), D ** -0.5), n((H * d, D), 2.0 * D ** -0.5), n((H * dv, D), D ** -0.5)
+            w[q + "f.b"], w[q + "lower"] = n((H * d,), 1.0, 1.0), torch.rand((H * d,), generator=g) * 0.95
+            w[q + "norm"], w[q + "o"] = n((dv,), 0.1, 1.0), n((D, H * dv), (H * dv) ** -0.5)
+        else:
+            H, G, d, dv = heads(w, q, m)
+            w[q + "q.norm"], w[q + "k.norm"] = n((H * d,), 0.1, 1.0), n((G * d,), 0.1, 1.0)
+            w[q + "rel"] = n((m["bias_rows"], H), 1.0)
+        mlp = entry.get("mlp")
+        if mlp is None:
+            continue
+        if mlp["kind"] == "dense":
+            ff(w, p + "mlp.", mlp["ff"])
+        else:
+            E = mlp["router"]["experts"]
+            for e in range(E):
+                ff(w, f"{p}mlp.e{e}.", mlp["expert"]["ff"])
+            w[p + "mlp.router"], w[p + "mlp.correction"] = n((E, D), 2.0 * D ** -0.5), n((E,), 0.05)
+            if mlp.get("shared"):
+                ff(w, p + "mlp.shared.", mlp["shared"]["ff"])
+    w["final.norm"], w["head"] = n((D,), 0.1), n((config["vocab"], D), D ** -0.5)
+    return w
+
+
+def model(w, config, tokens, margins=None):
+    """Float64 logits ``[T, vocab]`` from float32 (or rounded) weights."""
+    return forward(config, {k: v.double() for k, v in w.items()}, list(tokens), margins=margins)
+
+
+def greedy(w, config, prompt, n):
+    tokens, out = list(prompt), []
+    for _ in range(n):
+        out.append(int(model(w, config, tokens)[-1].argmax()))
+        tokens.append(out[-1])
+    return out
