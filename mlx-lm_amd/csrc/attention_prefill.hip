@@ -267,21 +267,31 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
                                  : (kt >= k_lo && kt + KT - 1 <= wave_q0 && wave_q0 + 31 < nq + pos0 &&
                                     (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
       if constexpr (SHAPED) {
-        // the score in its own units first: the cap and the table's term are no linear function of it
+        // the score in its own units first: the cap and the table's term are no linear function
+        // of it.  tanh(x) = 1 - 2 / (exp(2 x) + 1) through the hardware's exp2 and reciprocal (an
+        // exp2 that overflows gives the cap itself); a tile that lies wholly beyond the table's
+        // reach takes the table's last entry without a look-up.
         const int run_lo = sink ? 0 : k_lo, run_hi = sink ? sink_hi : k_hi;
         const float c1 = p.head_scale ? p.head_scale[h] : p.scale;
+        const float cap = p.softcap, cap_exp = cap > 0.f ? 2.0f * 1.4426950408889634f / cap : 0.f;
         const float* bias_row = p.dist_bias ? p.dist_bias + (size_t)h * p.n_dist : nullptr;
+        const int last = p.n_dist - 1;
+        const bool beyond = bias_row && wave_q0 - (kt + KT - 1) >= last;
+        const float beyond_bias = beyond ? bias_row[last] : 0.f;
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int o = 32 * s + 16 * (r >> 3) + (r & 7);
             const int key = kt + 8 * g + o;
-            const bool ok = q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first);
             float v = st[s][r] * c1;
-            if (p.softcap > 0.f) v = p.softcap * tanhf(v / p.softcap);
-            if (bias_row) v += bias_row[min(max(qpos - key, 0), p.n_dist - 1)];
+            if (cap > 0.f) v = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(v * cap_exp) + 1.0f));
+            if (beyond)
+              v += beyond_bias;
+            else if (bias_row)
+              v += bias_row[min(max(qpos - key, 0), last)];
             v = fmaf(v, 1.4426950408889634f, fmaf(slope2, (float)o, -far));
+            const bool ok = all_seen || (q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first));
             st[s][r] = ok ? v : -INFINITY;
             tmax = fmaxf(tmax, st[s][r]);
           }

@@ -10,7 +10,8 @@
 //                   option of head_prepare: the source's columns pass through it on their way in.
 //   head_prepare    a wave a (row, head): the head's `dim` columns from a float row (through the
 //                   convolution, where one is given); RMS norm over
-//                   the first `norm_dim` of them (times a weight of norm_dim values shared by all
+//                   the first `norm_dim` of them (or, with `norm_whole`, over all heads' columns at
+//                   once, with a weight for each) (times a weight of norm_dim values shared by all
 //                   heads, or none); rotation of the `rot_dims` columns from `rot_off` on by
 //                   position * inv_freq[i], pairs (2i, 2i + 1) or (i, i + rot_dims / 2), cos and
 //                   sin times `rot_mult`; then the head goes to `copies` places: copy c of head h
@@ -55,6 +56,10 @@ struct PrepareArgs {
   const int* block_table;
   int max_blocks, page_size;
   size_t page_stride;
+  // norm_whole > 0: the norm runs over the whole projection, the norm_whole columns from src_col
+  // on (all heads at once), with a weight for every one of them (norm_w [norm_whole]); every
+  // column of a head is normed.  Not together with a convolution.
+  int norm_whole;
 };
 
 template <typename T>
@@ -87,7 +92,13 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& a, long item, in
   }
   auto in = [&](int c) { return a.conv_w ? cv[c] : s[c]; };
   float rstd = 1.f;
-  if (a.norm_dim > 0) {
+  if (a.norm_whole > 0) {
+    // (every wave of the row adds up the whole projection itself: a few loads a lane)
+    const float* whole = a.src + (size_t)row * a.lds + a.src_col;
+    float q = 0.f;
+    for (int k = lane; k < a.norm_whole; k += 64) q += whole[k] * whole[k];
+    rstd = 1.0f / sqrtf(wave_sum(q) / (float)a.norm_whole + a.eps);
+  } else if (a.norm_dim > 0) {
     float q = 0.f;
     for (int k = lane; k < a.norm_dim; k += 64) {
       const float u = in(k);
@@ -108,7 +119,10 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& a, long item, in
     float v = 0.f;
     if (k < a.dim) {
       const int rel = k - a.rot_off;
-      auto at = [&](int c) { return c < a.norm_dim ? in(c) * rstd * (a.norm_w ? a.norm_w[c] : 1.f) : in(c); };
+      auto at = [&](int c) {
+        if (a.norm_whole > 0) return in(c) * rstd * (a.norm_w ? a.norm_w[h * a.src_stride + c] : 1.f);
+        return c < a.norm_dim ? in(c) * rstd * (a.norm_w ? a.norm_w[c] : 1.f) : in(c);
+      };
       v = at(k);
       if (rel >= 0 && rel < a.rot_dims) {
         int i, partner;
@@ -206,6 +220,9 @@ static int prepare_args_fit(const PrepareArgs& a) {
     FAIL("head_prepare: %d heads of %d columns, %d apart from column %d, in rows of %d", a.n_heads, a.dim, a.src_stride,
          a.src_col, a.lds);
   if (a.norm_dim < 0 || a.norm_dim > a.dim) FAIL("head_prepare: a norm over %d of %d columns", a.norm_dim, a.dim);
+  if (a.norm_whole < 0 || (a.norm_whole > 0 && (a.conv_w || a.norm_whole < (a.n_heads - 1) * a.src_stride + a.dim ||
+                                                 a.lds < a.src_col + a.norm_whole)))
+    FAIL("head_prepare: a norm over the whole projection of %d columns (no convolution; all heads inside)", a.norm_whole);
   if (a.rot_dims && (a.rot_dims % 2 || a.rot_off < 0 || a.rot_off + a.rot_dims > a.dim || !a.inv_freq || !a.positions))
     FAIL("head_prepare: %d turning columns from %d in a head of %d", a.rot_dims, a.rot_off, a.dim);
   if (a.copies < 1 || a.dst_fill < a.dim || a.dst_fill > a.dst_stride)

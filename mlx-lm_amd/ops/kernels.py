@@ -1071,7 +1071,7 @@ class PrepareArgs(ctypes.Structure):
                 ("conv_w", _vp), ("taps", _c_int), ("conv_channels", _c_int), ("conv_single", _c_int), ("conv_state", _vp),
                 ("conv_state_stride", _c_size_t), ("conv_offset", _c_size_t), ("seq_start", _vp), ("slot_ids", _vp),
                 ("token_req", _vp), ("block_table", _vp), ("max_blocks", _c_int), ("page_size", _c_int),
-                ("page_stride", _c_size_t)]
+                ("page_stride", _c_size_t), ("norm_whole", _c_int)]
 
 
 class ConvolutionAhead:
@@ -1113,7 +1113,9 @@ def head_prepare(dst, src, src_col, n_heads, dim, **options):
     by ``position * inv_freq[i]`` (pairs ``(2i, 2i + 1)`` with ``interleaved``, else ``(i, i +
     rot_dims / 2)``; cos and sin times ``rot_mult``); written to ``dst`` (float32 or bfloat16) at
     column ``dst_head[c, h] * dst_stride`` for each of ``copies`` copies (``h * dst_stride`` without
-    a table), with zeros from ``dim`` up to ``dst_fill`` columns.  ``conv`` (a ``ConvolutionAhead``):
+    a table), with zeros from ``dim`` up to ``dst_fill`` columns.  ``norm_whole = n``: the norm runs over
+    the ``n`` columns from ``src_col`` on, all heads at once, with ``norm_weight`` of ``n`` values, and
+    every column of a head is normed.  ``conv`` (a ``ConvolutionAhead``):
     the source's columns pass a causal convolution first.  ``dst`` may be a ``PagesOut``."""
     lib = build.load("head_prepare")
     a = _prepare_args(dst, src, src_col, n_heads, dim, **options)
@@ -1134,7 +1136,7 @@ def head_prepare_many(*calls):
 
 def _prepare_args(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=None, dst_fill=None, norm_dim=0,
                   norm_weight=None, eps=0.0, rot_off=0, rot_dims=0, inv_freq=None, rot_mult=1.0, interleaved=True,
-                  positions=None, dst_head=None, copies=1, conv=None):
+                  positions=None, dst_head=None, copies=1, conv=None, norm_whole=0):
     a = PrepareArgs()
     src_stride = dim if src_stride is None else src_stride
     n_rows = src.shape[0] if isinstance(dst, PagesOut) else dst.shape[0]
@@ -1143,10 +1145,10 @@ def _prepare_args(dst, src, src_col, n_heads, dim, src_stride=None, dst_stride=N
     a.src, a.src_col, a.src_stride = src.data_ptr(), int(src_col), int(src_stride)
     a.n_rows, a.n_heads, a.dim = n_rows, int(n_heads), int(dim)
     _need(src.shape[0] >= n_rows, "head_prepare: fewer source rows than rows of dst")
-    a.norm_dim, a.eps = int(norm_dim), float(eps)
+    a.norm_dim, a.eps, a.norm_whole = int(norm_dim), float(eps), int(norm_whole)
     if norm_weight is not None:
         _dev(norm_weight, "norm_weight", torch.float32)
-        _need(norm_weight.numel() == norm_dim, "head_prepare: norm_weight has norm_dim values")
+        _need(norm_weight.numel() == (norm_whole or norm_dim), "head_prepare: norm_weight has norm_dim values (norm_whole, for a norm over all heads)")
         a.norm_w = norm_weight.data_ptr()
     if rot_dims:
         _dev(inv_freq, "inv_freq", torch.float32)
@@ -1424,10 +1426,56 @@ def expert_tiles(y, x, w_gate, w_up, w_down, idx, weight, top, alloc, accumulate
 # a layer whose sublayers share one norm and whose outgoing stream is a sum over depth (csrc/parallel_block.hip)
 
 
-def norm_fanout(out, x, weight, eps, out32=None, copy_a=None, copy_b=None):
+class CanonArgs(ctypes.Structure):
+    """Mirror of ``CanonArgs`` in csrc/parallel_block.hip."""
+
+    _fields_ = [("w", _vp), ("taps", _c_int), ("state", _vp), ("state_stride", _c_size_t), ("state_offset", _c_size_t),
+                ("token_req", _vp), ("seq_start", _vp), ("slot_ids", _vp), ("mixed", _vp)]
+
+
+class InputConvolution:
+    """A causal convolution over time on a mixer's input, added to it: ``m_t = h_t + sum_j weight[:, j]
+    h_(t - taps + 1 + j)`` per channel over a request's own rows (``weight`` float32 ``[width, taps]``);
+    rows of earlier steps come from the request's row of ``state`` (``[taps - 1, width]`` from
+    ``offset`` on, the latest last).  ``mixed``: where ``m`` goes, ``[rows, width]`` in the compute dtype."""
+
+    def __init__(self, weight, state, offset, token_req, seq_start, slot_ids, mixed):
+        _dev(weight, "weight", torch.float32)
+        _dev(state, "state", torch.float32)
+        for name, t in (("token_req", token_req), ("seq_start", seq_start), ("slot_ids", slot_ids)):
+            _dev(t, name, torch.int32)
+        width, taps = weight.shape
+        _need(state.dim() == 2 and offset + (taps - 1) * width <= state.shape[1], "a convolution's state rows hold taps - 1 inputs of every channel")
+        _need(mixed.is_contiguous() and mixed.dtype in DT and mixed.shape[1] == width and token_req.numel() >= mixed.shape[0],
+              "the convolution's output is contiguous [rows, width]")
+        self.mixed, self.width = mixed, width
+        self._keep = (weight, state, token_req, seq_start, slot_ids)
+        c = self.c = CanonArgs()
+        c.w, c.taps, c.state, c.state_stride, c.state_offset = weight.data_ptr(), taps, state.data_ptr(), state.stride(0), int(offset)
+        c.token_req, c.seq_start, c.slot_ids, c.mixed = token_req.data_ptr(), seq_start.data_ptr(), slot_ids.data_ptr(), mixed.data_ptr()
+
+
+CANON_FUSED_MAX_WIDTH = 8192  # up to this width the norm's kernel keeps a row in registers and can run the convolution too
+
+
+def canon_rows(h, canon):
+    """``canon`` (an ``InputConvolution``) over the float32 rows ``h`` of a step of any shape; the
+    requests' state rows are not touched (``conv_state_update`` keeps the last inputs afterwards)."""
+    lib = build.load("parallel_block")
+    _dev(h, "h", torch.float32)
+    _need(h.dim() == 2 and h.shape[1] == canon.width and h.shape[0] >= canon.mixed.shape[0], "canon_rows: shapes")
+    rc = lib.canon_rows(_ptr(h), _c_int(canon.mixed.shape[0]), _c_int(canon.width), _c_int(DT[canon.mixed.dtype]),
+                        ctypes.byref(canon.c), _stream())
+    build.check(lib, rc, "canon_rows")
+    return canon.mixed
+
+
+def norm_fanout(out, x, weight, eps, out32=None, copy_a=None, copy_b=None, canon=None):
     """``out = x / sqrt(mean(x^2) + eps) * weight`` over the float32 rows ``x`` (``out``: float32 or
     bfloat16, contiguous); the same as float32 into ``out32``, and ``x`` itself into ``copy_a`` and
-    ``copy_b`` (contiguous float32 ``[rows, width]``), each where given."""
+    ``copy_b`` (contiguous float32 ``[rows, width]``), each where given.  ``canon`` (an
+    ``InputConvolution``, for a step in which every request brings one token): the convolution runs
+    here too, and every request's state row moves up by one."""
     lib = build.load("parallel_block")
     n, width = out.shape
     ldx = _f32_rows(x, "x", width)
@@ -1437,8 +1485,12 @@ def norm_fanout(out, x, weight, eps, out32=None, copy_a=None, copy_b=None):
         if t is not None:
             _dev(t, name, torch.float32)
             _need(t.is_contiguous() and tuple(t.shape) == (n, width), f"norm_fanout: {name} is contiguous [rows, width]")
+    if canon is not None:
+        _need(canon.width == width and canon.mixed.shape[0] == n and canon.mixed.dtype == out.dtype and width <= CANON_FUSED_MAX_WIDTH,
+              "norm_fanout: the convolution's rows are the norm's")
     rc = lib.norm_fanout(_ptr(x), _c_int(ldx), _ptr(weight), _c_float(eps), _c_int(n), _c_int(width), _ptr(out),
-                         _c_int(DT[out.dtype]), _ptr(out32), _ptr(copy_a), _ptr(copy_b), _stream())
+                         _c_int(DT[out.dtype]), _ptr(out32), _ptr(copy_a), _ptr(copy_b),
+                         ctypes.byref(canon.c) if canon is not None else None, _stream())
     build.check(lib, rc, "norm_fanout")
     return out
 

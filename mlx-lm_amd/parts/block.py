@@ -247,7 +247,7 @@ class SharedNormBlock(Block):
       layers: the one with ``depth = 0`` takes the memory, the sublayers add straight into ``Y``).
 
     The norm is an RMS norm (an ``rmsnorm`` part gives weight and eps).  Norm, convolution, the
-    sums and the weighted sum are 32-bit (csrc/parallel_block.hip, csrc/head_prepare.hip).  The
+    sums and the weighted sum are 32-bit (csrc/parallel_block.hip).  The
     run's state slot holds the convolution's inputs and, behind them, what a mixer that keeps
     state beside its pages (``wants_state``) asks for.  No counterpart in mlx_lm/models/gpt2.py,
     whose blocks have a norm for each sublayer and run them in turn (:98-108).
@@ -267,10 +267,8 @@ class SharedNormBlock(Block):
         self.width, self.eps = norm.width, norm.eps
         if self.width % 8:
             raise ValueError(f"width {self.width} must be a multiple of 8")
-        self.input_conv = ShortConvolution((self.width,), int(input_taps), (input_conv_name,), add_identity=True,
-                                           prefix=prefix) if input_taps else None
-        # (the convolution runs as ``head_prepare`` reads a row in pieces of at most 256 columns)
-        self.conv_piece = next(d for d in (256, 128, 64, 32, 16, 8) if self.width % d == 0)
+        # (the part holds the weights and knows the state's layout; the kernels are this arrangement's own)
+        self.input_conv = ShortConvolution((self.width,), int(input_taps), (input_conv_name,), prefix=prefix) if input_taps else None
         if depth is not None and not 0 <= depth < depth_total:
             raise ValueError(f"depth {depth} of {depth_total} layers")
         self.depth, self.depth_total, self.depth_name = depth, int(depth_total), self._name(depth_name)
@@ -331,16 +329,23 @@ class SharedNormBlock(Block):
             target = kept[self.depth + 1]
         mark = ctx.scratch_mark()
         u = ctx.scratch((T, W), ctx.dtype)
-        u32 = ctx.scratch((T, W), torch.float32) if self.input_conv is not None else None
+        um, u32, canon, conv = u, None, None, self.input_conv
+        if conv is not None:
+            um = ctx.scratch((T, W), ctx.dtype)
+            rows = state.state if conv.state_floats else conv.no_state
+            canon = kernels.InputConvolution(conv.weight, rows, 0, ctx.token_req, ctx.array("sequences.starts"), ctx.slot_ids, um)
+        # a step in which every request brings one token: norm, convolution and the state's move are one kernel
+        single = canon is not None and ctx.array("sequences.longest") == 1 and W <= kernels.CANON_FUSED_MAX_WIDTH
+        if canon is not None and not single:
+            u32 = ctx.scratch((T, W), torch.float32)
         # the norm; the stream itself goes where the sublayers add to it (and, first of all, to Y_0)
         kernels.norm_fanout(u, h, self.norm.weight, self.eps, out32=u32, copy_a=target,
-                            copy_b=kept[0] if self.depth == 0 else None)
-        um = u
-        if self.input_conv is not None:
-            um = ctx.scratch((T, W), ctx.dtype)
-            rows = state.state if state is not None else None
-            kernels.head_prepare(um, u32, 0, W // self.conv_piece, self.conv_piece, conv=self.input_conv.ahead(ctx, rows, 0))
-            self.input_conv.keep_inputs(ctx, u32, rows, 0)
+                            copy_b=kept[0] if self.depth == 0 else None, canon=canon if single else None)
+        if canon is not None and not single:
+            kernels.canon_rows(u32, canon)
+            if conv.state_floats:
+                kernels.conv_state_update(u32, 0, conv.taps, W, rows, 0, ctx.array("sequences.starts"), ctx.array("sequences.lens"),
+                                          ctx.slot_ids, ctx.n_requests)
         into = target if target is not None else h
         if self._mixer_state_need() is not None:
             self.mixer.forward(ctx, um, into, cache, writes_cache,

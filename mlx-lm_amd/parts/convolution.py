@@ -20,9 +20,8 @@ class ShortConvolution(_SequenceArrays, Part):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
 
-    def __init__(self, channels, taps, names, add_identity=False, prefix=""):
+    def __init__(self, channels, taps, names, prefix=""):
         super().__init__(prefix)
-        self.add_identity = bool(add_identity)  # ``y_t = u_t + sum_j ...``: one more on the current token's tap
         if taps < 1 or not channels or any(c <= 0 for c in channels) or len(channels) != len(names):
             raise ValueError(f"{taps} taps over channels {channels} of tensors {names}")
         self.channels, self.taps = [int(c) for c in channels], int(taps)
@@ -38,9 +37,6 @@ class ShortConvolution(_SequenceArrays, Part):
         import torch
 
         self.weight = torch.cat([tensors[n] for n in self.names]).contiguous()
-        if self.add_identity:
-            self.weight = self.weight.clone()
-            self.weight[:, -1] += 1.0
         # one tap keeps nothing between steps: the kernel still wants a base address, which it never reads
         self.no_state = self.weight.new_zeros((1, 1)) if not self.state_floats else None
 

@@ -36,7 +36,7 @@ class ScoredAttention(Mixer):
     ``gate``: the concatenated heads are multiplied by ``sigmoid(Wg x)`` (tensor ``g``) ahead of
     the output projection.
 
-    One product gives ``[q | k | v | g]`` as float32 rows; the norms are 32-bit; ``head_prepare``
+    One product gives ``[q | k | v | g]`` as float32 rows; the norms are 32-bit and run as ``head_prepare``
     lays the heads into the next head size that the fast attention kernels take (zeros beyond a
     head's own columns), keys and values straight into their pages.  The table of the distance
     term is made once, a float for every (head, distance) up to ``bias_far`` (beyond it the last
@@ -119,18 +119,14 @@ class ScoredAttention(Mixer):
         qc, kc, vc = self.q_cols, self.k_cols, self.v_cols
         u = ctx.scratch((T, qc + kc + vc + self.g_cols), torch.float32)
         kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
-        q_src, q_col, k_src, k_col = u, 0, u, qc
-        if self.whole_norm:
-            q_src, k_src = ctx.scratch((T, qc), torch.float32), ctx.scratch((T, kc), torch.float32)
-            kernels.rmsnorm(q_src, u, self.q_norm, self.eps)
-            kernels.rmsnorm(k_src, u[:, qc:], self.k_norm, self.eps)
-            q_col = k_col = 0
         q = ctx.scratch((T, H * hd), ctx.dtype)
         place = dict(dst_stride=hd, dst_fill=hd)
-        calls = [(q, q_src, q_col, H, d, place)]
+        q_norm = dict(norm_whole=qc, norm_weight=self.q_norm, eps=self.eps) if self.whole_norm else {}
+        k_norm = dict(norm_whole=kc, norm_weight=self.k_norm, eps=self.eps) if self.whole_norm else {}
+        calls = [(q, u, 0, H, d, dict(place, **q_norm))]
         if writes_cache:
             pages = [kernels.PagesOut(cache.kv, values, cache.block_table, ctx.token_req, ctx.positions) for values in (False, True)]
-            calls.append((pages[0], k_src, k_col, G, d, place))
+            calls.append((pages[0], u, qc, G, d, dict(place, **k_norm)))
             calls.append((pages[1], u, qc + kc, G, dv, place))
         gate = None
         if self.has_gate:
