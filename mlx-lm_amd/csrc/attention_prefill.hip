@@ -278,23 +278,40 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
         const int last = p.n_dist - 1;
         const bool beyond = bias_row && wave_q0 - (kt + KT - 1) >= last;
         const float beyond_bias = beyond ? bias_row[last] : 0.f;
+        const float raw_exp = c1 * cap_exp, cap2 = cap * 1.4426950408889634f;  // (the cap in units of log 2)
+        auto shaped = [&](float raw, int o, int key) {
+          const float away = fmaf(slope2, (float)o, -far);
+          if (cap > 0.f && !bias_row)  // cap2 * tanh = cap2 - 2 cap2 / (exp + 1)
+            return fmaf(__builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(raw * raw_exp) + 1.0f), -2.0f * cap2, cap2 + away);
+          float v = raw * c1;
+          if (cap > 0.f) v = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(v * cap_exp) + 1.0f));
+          if (beyond)
+            v += beyond_bias;
+          else if (bias_row)
+            v += bias_row[min(max(qpos - key, 0), last)];
+          return fmaf(v, 1.4426950408889634f, away);
+        };
+        if (all_seen) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+          for (int s = 0; s < 2; ++s)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int o = 32 * s + 16 * (r >> 3) + (r & 7);
-            const int key = kt + 8 * g + o;
-            float v = st[s][r] * c1;
-            if (cap > 0.f) v = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(v * cap_exp) + 1.0f));
-            if (beyond)
-              v += beyond_bias;
-            else if (bias_row)
-              v += bias_row[min(max(qpos - key, 0), last)];
-            v = fmaf(v, 1.4426950408889634f, fmaf(slope2, (float)o, -far));
-            const bool ok = all_seen || (q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first));
-            st[s][r] = ok ? v : -INFINITY;
-            tmax = fmaxf(tmax, st[s][r]);
-          }
+            for (int r = 0; r < 16; ++r) {
+              const int o = 32 * s + 16 * (r >> 3) + (r & 7);
+              st[s][r] = shaped(st[s][r], o, kt + 8 * g + o);
+              tmax = fmaxf(tmax, st[s][r]);
+            }
+        } else {
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int o = 32 * s + 16 * (r >> 3) + (r & 7);
+              const int key = kt + 8 * g + o;
+              const bool ok = q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first);
+              st[s][r] = ok ? shaped(st[s][r], o, key) : -INFINITY;
+              tmax = fmaxf(tmax, st[s][r]);
+            }
+        }
       } else if (all_seen) {
 #pragma unroll
         for (int s = 0; s < 2; ++s)
