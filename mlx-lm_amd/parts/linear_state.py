@@ -334,6 +334,7 @@ class LightningAttention(_SequenceArrays, Mixer):
         self.decay_values, self.eps = [float(d) for d in decay], float(eps)
         self.qk_width, self.v_width = n_heads * key_dim, n_heads * value_dim
         self.overwrite = False
+        self.projection_given = False  # a pair of parallel mixers makes both mixers' projections in one product
 
     def cache_need(self):
         return StateNeed((self.n_heads * self.key_dim * self.value_dim,), "float32")
@@ -347,20 +348,28 @@ class LightningAttention(_SequenceArrays, Mixer):
                 n("o"): TensorSpec((self.width, self.v_width), "matrix"),
                 n("norm"): TensorSpec((self.v_width,), "vector")}
 
+    def input_names(self):
+        """The tensors whose rows, in this order, are the projection that ``forward`` starts with."""
+        return [self._name(x) for x in ("q", "k", "v", "g")]
+
     def load(self, tensors):
         n = self._name
-        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in ("q", "k", "v", "g")]))
         self.out_w = _matrix(_padded_columns(tensors[n("o")]))
-        self.first_weight = self.in_w
+        if not self.projection_given:
+            self.in_w = _matrix(torch.cat([tensors[x] for x in self.input_names()]))
+            self.first_weight = self.in_w
         self.norm_w = tensors[n("norm")]
         self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=self.norm_w.device)
 
-    def forward(self, ctx, x, residual, cache, writes_cache=True):
+    def forward(self, ctx, x, residual, cache, writes_cache=True, rows=None):
+        """``rows``: the projection's float32 rows, where the caller has made them already."""
         T = x.shape[0]
         mark = ctx.scratch_mark()
         a, b = self.qk_width, 2 * self.qk_width
-        u = ctx.scratch((T, b + 2 * self.v_width), torch.float32)
-        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
+        u = rows
+        if u is None:
+            u = ctx.scratch((T, b + 2 * self.v_width), torch.float32)
+            kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
         kernels.silu_columns(u, 0, b + self.v_width)
         y = ctx.scratch((T, self.v_width), torch.float32)
         kernels.state_scan(y, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, cache.offset,
@@ -444,7 +453,8 @@ class ParallelMixers(Mixer):
     """Two mixers side by side that read the same input: ``left_scale * left(x) + right_scale *
     right(x)``.  The left one keeps the run's cache slot, the right one the run's state slot (the
     arrangement passes both on: ``wants_state``).  The two outputs are float32 rows and are summed
-    in float32."""
+    in float32.  Where both mixers start with a projection of ``x`` into float32 rows and name its
+    tensors (``input_names``), one product makes both projections and each mixer gets its columns."""
 
     can_overwrite = True
     wants_state = True
@@ -461,9 +471,22 @@ class ParallelMixers(Mixer):
             if getattr(m, "can_overwrite", False) and hasattr(m, "overwrite"):
                 m.overwrite = True
         self.graph_safe = all(getattr(m, "graph_safe", False) for m in (self.left, self.right))
+        # two mixers that start with a projection into float32 rows and say of which tensors
+        # (``input_names``) get both from one product
+        self.shared_projection = all(hasattr(m, "input_names") and hasattr(m, "projection_given") for m in (self.left, self.right))
+        if self.shared_projection:
+            self.left.projection_given = self.right.projection_given = True
+        self.in_w, self.in_cols = None, None
 
     def sub_parts(self):
         return (self.left, self.right)
+
+    def load(self, tensors):
+        if self.shared_projection:
+            parts = [[tensors[n] for n in m.input_names()] for m in (self.left, self.right)]
+            self.in_cols = [sum(t.shape[0] for t in ts) for ts in parts]
+            self.in_w = _matrix(torch.cat(parts[0] + parts[1]))
+            self.first_weight = self.in_w
 
     def cache_need(self):
         return self.left.cache_need()
@@ -479,12 +502,20 @@ class ParallelMixers(Mixer):
 
     def forward(self, ctx, x, residual, cache, writes_cache=True, state=None):
         mark = ctx.scratch_mark()
-        outs = []
-        for m, slot in ((self.left, cache), (self.right, state)):
+        outs, rows = [], (None, None)
+        if self.shared_projection:
+            T, (nl, nr) = x.shape[0], self.in_cols
+            u = ctx.scratch((T, nl + nr), torch.float32)
+            kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
+            rows = (u[:, :nl], u[:, nl:])
+        for m, slot, r in ((self.left, cache, rows[0]), (self.right, state, rows[1])):
             y = ctx.scratch(tuple(residual.shape), torch.float32)
             if not getattr(m, "overwrite", False):
                 y.zero_()
-            m.forward(ctx, x, y, slot, writes_cache)
+            if r is not None:
+                m.forward(ctx, x, y, slot, writes_cache, rows=r)
+            else:
+                m.forward(ctx, x, y, slot, writes_cache)
             outs.append(y)
         kernels.scaled_pair_sum(residual, self.left_scale, outs[0], self.right_scale, outs[1], accumulate=not self.overwrite)
         ctx.scratch_release(mark)

@@ -79,6 +79,7 @@ class ScoredAttention(Mixer):
         self.g_cols = n_heads * value_dim if self.has_gate else 0
         self.distance_bias = None
         self.overwrite = False
+        self.projection_given = False  # a pair of parallel mixers makes both mixers' projections in one product
 
     def cache_need(self):
         return CacheNeed(self.n_kv_heads, self.head_dim, self.window)
@@ -96,11 +97,15 @@ class ScoredAttention(Mixer):
             t[n("rel")] = TensorSpec((self.bias_rows, self.n_heads), "vector")
         return t
 
+    def input_names(self):
+        """The tensors whose rows, in this order, are the projection that ``forward`` starts with."""
+        return [self._name(x) for x in ("q", "k", "v") + (("g",) if self.has_gate else ())]
+
     def load(self, tensors):
         n, H, hd, dv = self._name, self.n_heads, self.head_dim, self.value_dim
-        names = ("q", "k", "v") + (("g",) if self.has_gate else ())
-        self.in_w = _matrix(torch.cat([tensors[n(x)] for x in names]))
-        self.first_weight = self.in_w
+        if not self.projection_given:
+            self.in_w = _matrix(torch.cat([tensors[x] for x in self.input_names()]))
+            self.first_weight = self.in_w
         # the output projection meets heads of ``head_dim`` columns: zero columns beyond a head's values
         o = tensors[n("o")].view(self.width, H, dv)
         self.out_w = _matrix(torch.cat([o, o.new_zeros(self.width, H, hd - dv)], 2).reshape(self.width, H * hd))
@@ -113,12 +118,15 @@ class ScoredAttention(Mixer):
             rows = torch.tensor([distance_bucket(d, self.bias_rows, self.bias_far) for d in range(n_dist)])
             self.distance_bias = rel[rows].t().contiguous().to(tensors[n("rel")].device)
 
-    def forward(self, ctx, x, residual, cache, writes_cache=True):
+    def forward(self, ctx, x, residual, cache, writes_cache=True, rows=None):
+        """``rows``: the projection's float32 rows, where the caller has made them already."""
         T, H, G, hd, d, dv = x.shape[0], self.n_heads, self.n_kv_heads, self.head_dim, self.key_dim, self.value_dim
         mark = ctx.scratch_mark()
         qc, kc, vc = self.q_cols, self.k_cols, self.v_cols
-        u = ctx.scratch((T, qc + kc + vc + self.g_cols), torch.float32)
-        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
+        u = rows
+        if u is None:
+            u = ctx.scratch((T, qc + kc + vc + self.g_cols), torch.float32)
+            kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
         q = ctx.scratch((T, H * hd), ctx.dtype)
         place = dict(dst_stride=hd, dst_fill=hd)
         q_norm = dict(norm_whole=qc, norm_weight=self.q_norm, eps=self.eps) if self.whole_norm else {}
