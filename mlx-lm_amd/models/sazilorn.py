@@ -6,7 +6,7 @@ layers
 
     ``u = N(x; 1 + w)``,  ``Y_(i+1) = x + mixer(u + conv(u)) + ff(u)``,  ``x <- sum_(j <= i+1) a_i[j] Y_j``
 
-with an RMS norm whose weight is stored around zero, a short causal convolution over time on what
+with an RMS norm whose tensor holds the scale's difference from one, a short causal convolution over time on what
 the mixer reads, and ``Y_0`` the embedding's output; the model's norm and an untied head.  Mixers:
 
 * ``parallel``: two mixers on the same input, summed with two constants: softmax attention with
@@ -14,7 +14,7 @@ the mixer reads, and ``Y_0`` the embedding's output; the model's norm and an unt
   concatenated heads (``scored_attention``), beside linear attention with a fixed decay per
   head, silu on queries, keys and values, one norm over all heads and a sigmoid gate
   (``lightning_attention``);
-* ``hgrn2``: linear attention whose forget gate, bounded below, also decides what is written
+* ``hgrn2``: linear attention with a forget gate per key channel that has a floor, and whose complement is the key
   (``forget_gate_attention``);
 * ``attention``: softmax attention with grouped key heads, queries and keys normed over their
   whole projection, and a learned bias by bucketed distance (``scored_attention``).

@@ -311,8 +311,8 @@ class LightningAttention(_SequenceArrays, Mixer):
         ``S_t = decay_h S_(t-1) + k_t v_t^T``,   ``o_t = S_t^T q_t``
 
     with ``q = silu(Wq x)``, ``k = silu(Wk x)`` (``n_heads x key_dim``), ``v = silu(Wv x)`` (``n_heads x
-    value_dim``) and no other scale.  The concatenated heads are RMS-normed together with the weight
-    ``norm`` (``n_heads * value_dim`` values), multiplied by ``sigmoid(Wg x)`` and projected by
+    value_dim``); nothing else is scaled.  The heads, side by side, pass one RMS norm with the weight
+    ``norm`` (``n_heads * value_dim`` values), are multiplied by ``sigmoid(Wg x)`` and projected by
     ``Wo``.  ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start) is the
     request's state.  One product gives ``[q | k | v | g]`` as float32 rows; the activations, the
     recurrence, the norm and the gate are 32-bit (csrc/state_gates.hip, csrc/linear_state.hip).
@@ -383,13 +383,13 @@ class LightningAttention(_SequenceArrays, Mixer):
 
 
 class ForgetGateAttention(_SequenceArrays, Mixer):
-    """Linear attention in which the forget gate also decides what is written (HGRN2):
+    """Linear attention whose key is the complement of its forget gate (HGRN2):
 
         ``S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T``,   ``o_t = S_t^T q_t``
 
     with ``q = silu(Wq x)`` (``n_heads x key_dim``), ``v = Wv x`` (``n_heads x value_dim``) and, per
     head and key channel, ``f = l + (1 - l) sigmoid(Wf x + b)`` with the floor ``l`` from the tensor
-    ``lower``; there is no key projection and no other scale.  Each head's ``o`` is RMS-normed over
+    ``lower``; the keys come from the gate alone and nothing is scaled.  Each head's ``o`` is RMS-normed over
     ``value_dim`` with the weight ``norm`` (shared by the heads), the heads are concatenated and
     projected by ``Wo``.  ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start)
     is the request's state.  One product gives ``[q | z | v]`` as float32 rows; ``1 - f`` (made as

@@ -59,7 +59,7 @@ class LayerNorm(Norm):
 
 class RMSNorm(Norm):
     """``x / sqrt(mean(x^2) + eps) * weight``: no mean is taken off, eps sits inside the root.
-    With ``offset`` the scale is ``offset + weight`` (a weight stored around zero with ``offset = 1``).
+    With ``offset`` the scale is ``offset + weight`` (a tensor that holds the scale's difference from one: ``offset = 1``).
 
     Reads the float32 residual stream, computes in float32, writes the compute dtype (``rows``:
     only those rows, for the rows whose logits are wanted).  An arrangement that norms after
@@ -81,7 +81,7 @@ class RMSNorm(Norm):
         return {self.weight_name: TensorSpec((self.width,), "vector")}
 
     def load(self, tensors):
-        # ``offset``: the tensor is stored around zero and the scale is ``offset + tensor`` (float32)
+        # ``offset``: the scale is ``offset + tensor`` (float32)
         self.weight = tensors[self.weight_name] + self.offset if self.offset else tensors[self.weight_name]
 
     def make_native(self):

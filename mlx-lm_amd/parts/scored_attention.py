@@ -29,7 +29,7 @@ class ScoredAttention(Mixer):
 
     * ``softcap``: ``softcap * tanh(score / softcap)``;
     * ``bias_rows`` (with ``bias_far``): a learned term ``rel[bucket(i - j), h]`` from the tensor
-      ``rel`` ``[bias_rows, n_heads]`` is added (``distance_bucket``); ``scale`` does not multiply it.
+      ``rel`` ``[bias_rows, n_heads]`` is added (``distance_bucket``), after the scaling.
 
     ``whole_norm``: queries and keys are RMS-normed over their whole projection (all heads at once,
     before the split into heads) with plain weights ``q.norm`` and ``k.norm`` of that size.

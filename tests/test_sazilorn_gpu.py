@@ -37,10 +37,10 @@ CONFIGS = {
         _dense(_attention(4, 2, 8, 24, 7, 1000), 12),
         _moe(_hgrn2(3, 8, 24), 4, 4, 12, shared=20)], eps=1e-3),
     # wider, for bfloat16: heads of 64
-    "C": _config(128, 300, 512, 3, [
-        _dense(_parallel(_softmax(4, 2, 64, 64, softcap=20.0), 2, 32, 32, [0.6, 0.999]), 96),
-        _moe(_hgrn2(2, 32, 64), 8, 3, 32, shared=32, scale=2.0),
-        _dense(_attention(4, 1, 64, 64, 32, 120), 96),
+    "C": _config(128, 300, 512, 2, [
+        _dense(_parallel(_softmax(4, 2, 64, 64, softcap=15.0), 2, 64, 32, [0.7, 0.995]), 96),
+        _moe(_hgrn2(2, 32, 64), 6, 2, 32, shared=32, scale=1.7),
+        _dense(_attention(4, 2, 64, 64, 24, 100), 96),
         _moe(_parallel(_softmax(2, 1, 64, 32, softcap=30.0), 4, 16, 16, [0.9, 0.95, 0.99, 0.5]), 4, 2, 48),
         _hgrn2(4, 16, 32)]),
 }
